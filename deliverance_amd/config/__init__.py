@@ -1,7 +1,8 @@
 from .specs import (AttentionSpec, ConfigError, DenseFeedForwardSpec, LayerCall, LayerSpec,
                     ModelConfig, NormSpec, PositionSpec)
 from .gpt2 import Gpt2Config
+from .virudra import VirudraConfig
 from .engine_config import EngineConfig
 
 __all__ = ["AttentionSpec", "ConfigError", "DenseFeedForwardSpec", "LayerCall", "LayerSpec",
-           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "EngineConfig"]
+           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "VirudraConfig", "EngineConfig"]

@@ -23,10 +23,14 @@ class ConfigError(ValueError):
 
 @dataclass(frozen=True)
 class NormSpec:
-    kind: str            # "layernorm" (others are added through parts.register_norm)
+    """``kind == "layernorm"``: mean and variance, gain and optional bias.  ``kind == "rmsnorm"``: the row
+    divided by its root mean square (eps inside the root) times ``gain_offset + weight``; a gain that is
+    stored around zero has ``gain_offset`` 1.  Others are added through ``parts.register_norm``."""
+    kind: str
     width: int
     eps: float
     bias: bool = True
+    gain_offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -43,17 +47,48 @@ class PositionSpec:
 
 
 @dataclass(frozen=True)
+class DistanceBiasSpec:
+    """A learned value per head that is added to a score by the distance n = i - j >= 0 between query and
+    key (after the scale; the scale does not multiply it).  The table has ``n_buckets`` rows: distances
+    below ``n_buckets // 2`` have a row each, larger ones share rows in steps that grow like a logarithm
+    up to ``max_distance``, from where the last row is used:
+
+        half = n_buckets // 2
+        bucket(n) = n                                                            for n < half
+                  = min(n_buckets - 1,
+                        half + floor(ln(n / half) / ln(max_distance / half) * (n_buckets - half)))   else
+    """
+    n_buckets: int
+    max_distance: int
+
+
+@dataclass(frozen=True)
+class QueryTemperatureSpec:
+    """Queries at position p are multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``: scores sharpen
+    as a sequence grows, in steps of ``every`` positions."""
+    coef: float
+    every: int
+
+
+@dataclass(frozen=True)
 class AttentionSpec:
     kind: str            # "attention"
     width: int           # model width E
     n_heads: int
     n_kv_heads: int
-    head_dim: int
+    head_dim: int        # per-head size of queries and keys
     scale: float         # multiplies q.k before the softmax
     qkv_bias: bool = True
     out_bias: bool = True
     window: Optional[int] = None     # None: every earlier key; w: the last w keys
     position: Optional[PositionSpec] = None  # acts on q and k (none for learned tables)
+    v_head_dim: Optional[int] = None         # per-head size of values; None: head_dim
+    distance_bias: Optional[DistanceBiasSpec] = None
+    query_temperature: Optional[QueryTemperatureSpec] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -63,6 +98,30 @@ class DenseFeedForwardSpec:
     inner: int
     activation: str      # "gelu_new" | "gelu" | "gelu_pytorch_tanh" | "relu" | "silu"
     bias: bool = True
+
+
+@dataclass(frozen=True)
+class GatedFeedForwardSpec:
+    """``down(act(gate h) * (up h))``, no biases."""
+    kind: str            # "gated"
+    width: int
+    inner: int
+    activation: str
+
+
+@dataclass(frozen=True)
+class ExpertsFeedForwardSpec:
+    """``n_experts`` gated feed-forwards of ``inner`` columns, of which every token uses ``top``; the output is
+    the weighted sum of theirs.  ``router == "token_table"``: a table [vocab, top] of integers names each
+    token id's experts (a row's entries differ), each with weight 1 / top."""
+    kind: str            # "experts"
+    width: int
+    inner: int
+    n_experts: int
+    top: int
+    activation: str
+    router: str = "token_table"
+    vocab_size: int = 0
 
 
 @dataclass(frozen=True)
@@ -118,6 +177,8 @@ class ModelConfig:
     embed_scale: float = 1.0        # multiplies the token embedding before positions are added
     # logits are divided by it (the reference's logitMultiplier, AbstractGeneratorSampler.java:117-120)
     logit_multiplier: float = 1.0
+    # logits <- cap * tanh(logits / cap) when positive
+    logit_softcap: float = 0.0
 
     @property
     def n_cache_slots(self) -> int:

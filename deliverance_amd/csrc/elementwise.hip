@@ -1,0 +1,41 @@
+// Small elementwise kernels.
+//   da_gated_act   mid[r, j] = act(gu[r, j]) * gu[r, inner + j]     the two halves of a fused gate | up product
+//   da_softcap     v <- cap * tanh(v / cap)                         in place, 32-bit
+#include "common.h"
+
+template <typename T, bool FAST>
+__global__ void gated_act_kernel(const T* __restrict__ gu, int ld, T* __restrict__ mid, int ldm, int R, int inner, int act) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)R * inner) return;
+  const int r = (int)(i / inner), j = (int)(i % inner);
+  const float g = to_f32(gu[(size_t)r * ld + j]), u = to_f32(gu[(size_t)r * ld + inner + j]);
+  from_f32(&mid[(size_t)r * ldm + j], (FAST ? apply_act_bf16(g, act) : apply_act(g, act)) * u);
+}
+
+extern "C" int da_gated_act(const void* gu, int ld, int dtype, void* mid, int ldm, int R, int inner, int act, void* stream) {
+  DA_REQUIRE(R >= 0 && inner > 0 && ld >= 2 * inner && ldm >= inner, "gated_act: bad sizes R=%d inner=%d", R, inner);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gated_act: unknown activation %d", act);
+  if (R == 0) return 0;
+  const long n = (long)R * inner;
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL((gated_act_kernel<bf16_t, true>), dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)gu, ld, (bf16_t*)mid, ldm, R, inner, act);
+  else
+    hipLaunchKernelGGL((gated_act_kernel<float, false>), dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const float*)gu, ld, (float*)mid, ldm, R, inner, act);
+  DA_CHECK_LAUNCH("gated_act");
+  return 0;
+}
+
+__global__ void softcap_kernel(float* __restrict__ v, long n, float cap) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[i] = cap * tanhf(v[i] / cap);
+}
+
+extern "C" int da_softcap(float* v, long n, float cap, void* stream) {
+  DA_REQUIRE(n >= 0 && cap > 0.f, "softcap: bad size or cap");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(softcap_kernel, dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, v, n, cap);
+  DA_CHECK_LAUNCH("softcap");
+  return 0;
+}

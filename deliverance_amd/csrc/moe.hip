@@ -1,0 +1,238 @@
+// Feed-forward layers made of experts: every token's rows go through `top` of `n_experts` small gated
+// feed-forwards, and the results are added with weights.
+//
+//   da_moe_route    from each token's expert ids (read from a table by token id, or given) to a layout in
+//                   which every expert's (token, choice) pairs lie together: pairs get slots, an expert's
+//                   slots start at a multiple of `tile` rows, so that a tile of rows has one expert
+//   da_moe_gated    mid[slot] = act(Wg_e a[row]) * (Wu_e a[row])      (plain kernel, any dtype)
+//   da_moe_down     out[slot] = Wd_e mid[slot]                        (plain kernel, 32-bit out)
+//   da_moe_combine  y[n] (+)= sum_k weight_k * out[slot(n, k)]        k ascending
+//
+// Everything the grid depends on comes from the step's shape (tokens x top, experts); which tiles are
+// used is decided on the device, so a step can be recorded.  A pair's result does not depend on its slot:
+// sums over k run in the same order for every row.  Expert weights are stacked: gate | up as
+// [n_experts][2 F][K] (gate rows first), down as [n_experts][width][F].
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+
+__global__ void __launch_bounds__(1024)
+moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int vocab, const int* __restrict__ ids,
+                 int N, int top, int n_experts, int tile, int* __restrict__ slot_of_pair,
+                 int* __restrict__ row_of_slot, int* __restrict__ tile_expert, int P_cap, int T_cap) {
+  __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], cursor[MOE_MAX_EXPERTS];
+  const int t = threadIdx.x, nt = blockDim.x;
+  const int P = N * top;
+  for (int e = t; e < n_experts; e += nt) counts[e] = cursor[e] = 0;
+  for (int i = t; i < P_cap; i += nt) row_of_slot[i] = -1;
+  for (int i = t; i < T_cap; i += nt) tile_expert[i] = -1;
+  __syncthreads();
+  auto expert_of = [&](int i) -> int {
+    int e;
+    if (table) {
+      const int tok = tokens[i / top];
+      e = (tok >= 0 && tok < vocab) ? table[(size_t)tok * top + i % top] : -1;
+    } else {
+      e = ids[i];
+    }
+    return (e >= 0 && e < n_experts) ? e : -1;
+  };
+  for (int i = t; i < P; i += nt) {
+    const int e = expert_of(i);
+    if (e >= 0) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (t == 0) {
+    int run = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      start[e] = run;
+      const int tiles = (counts[e] + tile - 1) / tile;
+      for (int k = 0; k < tiles; ++k) tile_expert[run / tile + k] = e;
+      run += tiles * tile;
+    }
+  }
+  __syncthreads();
+  for (int i = t; i < P; i += nt) {
+    const int e = expert_of(i);
+    int slot = -1;
+    if (e >= 0) {
+      slot = start[e] + atomicAdd(&cursor[e], 1);
+      row_of_slot[slot] = i / top;
+    }
+    slot_of_pair[i] = slot;
+  }
+}
+
+extern "C" int da_moe_route(const int* tokens, const int* table, int vocab, const int* ids, int N, int top,
+                            int n_experts, int tile, int* slot_of_pair, int* row_of_slot, int* tile_expert, int P_cap,
+                            int T_cap, void* stream) {
+  DA_REQUIRE(N >= 0 && top > 0 && n_experts > 0 && tile > 0, "moe_route: bad sizes");
+  DA_REQUIRE(n_experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, %d are taken", n_experts, MOE_MAX_EXPERTS);
+  DA_REQUIRE((table != nullptr && tokens != nullptr) != (ids != nullptr), "moe_route: a table with tokens, or expert ids");
+  DA_REQUIRE(T_cap >= da_ceil_div((long)N * top, tile) + n_experts && P_cap >= T_cap * tile,
+             "moe_route: the slot space (%d rows, %d tiles) is too small for %d pairs", P_cap, T_cap, N * top);
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, tokens, table, vocab, ids, N, top,
+                     n_experts, tile, slot_of_pair, row_of_slot, tile_expert, P_cap, T_cap);
+  DA_CHECK_LAUNCH("moe_route");
+  return 0;
+}
+
+// ---- plain grouped products: tiles of 64 x 64, sums in two levels as the plain product has them ------------
+#define MT 64
+#define MBK 16
+#define MCHUNK 8
+
+// GATED: two products (gate and up rows of the expert's stacked matrix), out = act(g) * u in T;
+// else one product, 32-bit out.  GATHER: row r of the tile is a[row_of_slot[slot]], else a[slot].
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
+                       const int* __restrict__ tile_expert, const T* __restrict__ w, void* __restrict__ out, int ldo,
+                       int K, int F, int act) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  __shared__ float As[MBK][MT + 4];
+  __shared__ float Ws[GATED ? 2 : 1][MBK][MT + 4];
+  __shared__ int srow[MT];
+  const int t = threadIdx.x;
+  const int tx = t % 16, ty = t / 16;
+  const int m0 = blockIdx.y * MT, n0 = blockIdx.x * MT;
+  const int lrow = t / 4, lk = (t % 4) * 4;
+  if (t < MT) srow[t] = row_of_slot[m0 + t];
+  __syncthreads();
+  const T* wg = w + (size_t)e * (GATED ? 2 : 1) * F * K;
+  const T* wu = wg + (size_t)F * K;
+  float acc[GATED ? 2 : 1][4][4], part[GATED ? 2 : 1][4][4];
+#pragma unroll
+  for (int g = 0; g < (GATED ? 2 : 1); ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[g][i][j] = part[g][i][j] = 0.f;
+  const int arow = GATED ? srow[lrow] : (srow[lrow] >= 0 ? m0 + lrow : -1);
+  int slab = 0;
+  for (int k0 = 0; k0 < K; k0 += MBK) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int k = k0 + lk + x;
+      const int wn = n0 + lrow;
+      As[lk + x][lrow] = (arow >= 0 && k < K) ? to_f32(a[(size_t)arow * lda + k]) : 0.f;
+      Ws[0][lk + x][lrow] = (wn < F && k < K) ? to_f32(wg[(size_t)wn * K + k]) : 0.f;
+      if (GATED) Ws[1][lk + x][lrow] = (wn < F && k < K) ? to_f32(wu[(size_t)wn * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < MBK; ++k) {
+      float av[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int g = 0; g < (GATED ? 2 : 1); ++g) {
+        float wv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wv[j] = Ws[g][k][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) part[g][i][j] = fmaf(av[i], wv[j], part[g][i][j]);
+      }
+    }
+    if (++slab == MCHUNK) {
+      slab = 0;
+#pragma unroll
+      for (int g = 0; g < (GATED ? 2 : 1); ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[g][i][j] += part[g][i][j];
+            part[g][i][j] = 0.f;
+          }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int g = 0; g < (GATED ? 2 : 1); ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[g][i][j] += part[g][i][j];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (srow[r] < 0) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= F) continue;
+      const size_t o = (size_t)(m0 + r) * ldo + n;
+      if (GATED) {
+        // the gate is rounded as a product of its own would be before the activation sees it
+        if (DTypeOf<T>::value == DA_BF16)
+          from_f32(&((T*)out)[o], apply_act_bf16(acc[0][i][j], act) * acc[1][i][j]);
+        else
+          from_f32(&((T*)out)[o], apply_act(acc[0][i][j], act) * acc[1][i][j]);
+      } else {
+        ((float*)out)[o] = acc[0][i][j];
+      }
+    }
+  }
+}
+
+extern "C" int da_moe_gated_ref(const void* a, int lda, int dtype, const int* row_of_slot, const int* tile_expert,
+                                const void* w, void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
+  DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_ref: bad sizes");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "moe_gated_ref: unknown activation %d", act);
+  if (T_cap == 0) return 0;
+  dim3 grid(da_ceil_div(F, MT), T_cap);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, true>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
+                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act);
+  else
+    hipLaunchKernelGGL((moe_product_ref_kernel<float, true>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
+                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act);
+  DA_CHECK_LAUNCH("moe_gated_ref");
+  return 0;
+}
+
+extern "C" int da_moe_down_ref(const void* mid, int ldm, int dtype, const int* row_of_slot, const int* tile_expert,
+                               const void* w, float* out, int ldo, int T_cap, int F, int width, void* stream) {
+  DA_REQUIRE(T_cap >= 0 && F > 0 && width > 0 && ldm >= F && ldo >= width, "moe_down_ref: bad sizes");
+  if (T_cap == 0) return 0;
+  dim3 grid(da_ceil_div(width, MT), T_cap);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, false>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F, width, 0);
+  else
+    hipLaunchKernelGGL((moe_product_ref_kernel<float, false>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const float*)mid, ldm, row_of_slot, tile_expert, (const float*)w, out, ldo, F, width, 0);
+  DA_CHECK_LAUNCH("moe_down_ref");
+  return 0;
+}
+
+// y[n] (+)= sum_k weight(n, k) * out[slot_of_pair[n * top + k]]; weights: per pair, or one for all
+__global__ void moe_combine_kernel(const float* __restrict__ out, int ldo, const int* __restrict__ slot_of_pair,
+                                   const float* __restrict__ weights, float uniform, int top, float* __restrict__ y,
+                                   int ldy, int N, int width, int accumulate) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)N * width) return;
+  const int n = (int)(i / width), c = (int)(i % width);
+  float s = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const int slot = slot_of_pair[n * top + k];
+    if (slot >= 0) s += (weights ? weights[n * top + k] : uniform) * out[(size_t)slot * ldo + c];
+  }
+  float* dst = y + (size_t)n * ldy + c;
+  *dst = accumulate ? *dst + s : s;
+}
+
+extern "C" int da_moe_combine(const float* out, int ldo, const int* slot_of_pair, const float* weights, float uniform,
+                              int top, float* y, int ldy, int N, int width, int accumulate, void* stream) {
+  DA_REQUIRE(N >= 0 && width > 0 && top > 0 && ldo >= width && ldy >= width, "moe_combine: bad sizes");
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(da_ceil_div((long)N * width, 256)), dim3(256), 0, (hipStream_t)stream, out,
+                     ldo, slot_of_pair, weights, uniform, top, y, ldy, N, width, accumulate);
+  DA_CHECK_LAUNCH("moe_combine");
+  return 0;
+}

@@ -10,7 +10,7 @@ to each other for the attention kernels.  All slots of a group live in one alloc
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -31,20 +31,26 @@ class DeviceCache:
         for slot in sorted(needs):
             need = needs[slot]
             if isinstance(need, KVNeed):
-                by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window), []).append(slot)
+                by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window, need.v_head_dim), []).append(slot)
             elif isinstance(need, StateNeed):
                 state_specs.append(StateSpec(slot, need.elems))
                 state_needs[slot] = need
             else:
                 raise TypeError(f"cache slot {slot}: unknown kind of need {need!r}")
-        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w), slots in by_shape.items()]
+        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w, _), slots in by_shape.items()]
+        # per group: the per-head size of values where it differs from the keys' (None: the same)
+        self.v_head_dims: List[Optional[int]] = [dv if dv != d else None for (_, d, _, dv) in by_shape]
         self.n_pages = -(-max_cached_tokens // page_size)
         self.group_of_slot: Dict[int, int] = {}
         self.kv: Dict[int, torch.Tensor] = {}
         self._group_tensors: List[torch.Tensor] = []
         for g, spec in enumerate(self.groups):
-            t = torch.empty((len(spec.slots), self.n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
-                            dtype=dtype, device=self.device)
+            dv = self.v_head_dims[g]
+            # keys and values of one size: [pages, 2, Hkv, page, D]; values of their own size: a page is
+            # Hkv * page * D keys, then Hkv * Dv * page values, [pages, Hkv * page * (D + Dv)]
+            shape = (2, spec.n_kv_heads, page_size, spec.head_dim) if dv is None else \
+                (spec.n_kv_heads * page_size * (spec.head_dim + dv),)
+            t = torch.empty((len(spec.slots), self.n_pages, *shape), dtype=dtype, device=self.device)
             # Pages are never cleared when they change hands (what a request may see is decided
             # by its length); the pool starts as NaN so that a read of a row nobody wrote shows.
             t.fill_(float("nan"))
@@ -76,7 +82,8 @@ class DeviceCache:
 
     def bytes_per_token(self) -> int:
         el = torch.empty((), dtype=self.dtype).element_size()
-        return sum(len(g.slots) * 2 * g.n_kv_heads * g.head_dim * el for g in self.groups)
+        return sum(len(g.slots) * g.n_kv_heads * (g.head_dim + (dv or g.head_dim)) * el
+                   for g, dv in zip(self.groups, self.v_head_dims))
 
     def state_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.state.values())
@@ -90,6 +97,7 @@ class DeviceCache:
     def tokens_for_budget(needs: Dict[int, object], dtype: torch.dtype, budget_bytes: int, n_state_slots: int = 0) -> int:
         """How many tokens' keys and values fit into ``budget_bytes`` once the state slots are paid for."""
         el = torch.empty((), dtype=dtype).element_size()
-        per_token = sum(2 * n.n_kv_heads * n.head_dim * el for n in needs.values() if isinstance(n, KVNeed))
+        per_token = sum(n.n_kv_heads * (n.head_dim + (n.v_head_dim or n.head_dim)) * el
+                        for n in needs.values() if isinstance(n, KVNeed))
         left = budget_bytes - DeviceCache.state_bytes_for(needs, n_state_slots)
         return max(0, left // max(per_token, 1))

@@ -120,6 +120,8 @@ class NativeStep:
             at, ff = blk.mixer, blk.feed_forward
             if type(at) is not CausalSelfAttention or at.position is not None or at.head_dim % 16 or at.head_dim > 256:
                 return False
+            if at.extras:          # a bias by distance, a query temperature, values of their own size
+                return False
             if (type(blk.pre_mixer_norm) is not LayerNorm or blk.post_mixer_norm is not None or blk.post_ff_norm is not None
                     or blk.post_block_norm is not None or blk.residual_multiplier != 1.0):
                 return False

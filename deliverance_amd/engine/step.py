@@ -173,7 +173,8 @@ class StepRunner:
         self._staging: Optional[torch.Tensor] = None     # pinned host buffer for the step's integers
         self._staging_dev: Optional[torch.Tensor] = None
         self._copied = None
-        self.max_blocks_cap = -(-model.config.max_positions // cache.page_size)
+        # a request never holds more pages than the pool has, whatever the model's position limit
+        self.max_blocks_cap = min(-(-model.config.max_positions // cache.page_size), max(1, cache.n_pages))
         self.last_ctx: Optional[StepContext] = None
         self.use_graphs = use_graphs and model.graph_safe
         self.max_graph_batch = max_graph_batch

@@ -90,6 +90,16 @@ _ARGTYPES = {
     "da_can_fuse_ln": [_I, _I, _I],
     "da_run_step": [_VP, _VP],
     "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
+    "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
+    "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
+    "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _VP],
+    "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
+    "da_softcap": [_VP, ctypes.c_long, _F, _VP],
+    "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP],
+    "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
+    "da_moe_combine": [_VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _I, _I, _VP],
 }
 _LIB = None
 
@@ -255,6 +265,153 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, gain_offset: float, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = x[rows[r] or r] / sqrt(mean(x^2) + eps) * (gain_offset + weight), in 32-bit."""
+    _dev(x, weight, out, rows)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2, "rmsnorm: x must be contiguous float32 [N, E]")
+    E, R = x.shape[1], out.shape[0]
+    _need(out.is_contiguous() and out.dim() == 2 and out.shape[1] == E, "rmsnorm: out must be contiguous [R, E]")
+    _need(weight.numel() == E and weight.is_contiguous(), "rmsnorm: the gain's length differs from E")
+    if rows is None:
+        _need(R <= x.shape[0], "rmsnorm: more output rows than input rows")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= R, "rmsnorm: rows must be int32 with R entries")
+    with _timed("rmsnorm", R * E * (4 + out.element_size()) + _nbytes(weight), 4 * R * E, "fp32"):
+        _check(_lib().da_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _dt(weight), float(gain_offset), float(eps),
+                                 _ptr(out), _dt(out), R, E, _stream()))
+    return out
+
+
+def rmsnorm_add(src: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, gain_offset: float, eps: float,
+                next_weight: Optional[torch.Tensor] = None, next_out: Optional[torch.Tensor] = None) -> None:
+    """x += rms(src) with ``weight``; with ``next_weight``, ``next_out = rms(x)`` of the new x in the same pass
+    (the norm behind a part, the residual addition and the norm in front of the next part)."""
+    _dev(src, weight, x, next_weight, next_out)
+    _need(src.dtype == torch.float32 and x.dtype == torch.float32 and src.is_contiguous() and x.is_contiguous()
+          and src.dim() == 2 and src.shape == x.shape, "rmsnorm_add: src and x must be contiguous float32 of one shape")
+    R, E = x.shape
+    _need(weight.numel() == E and weight.is_contiguous(), "rmsnorm_add: the gain's length differs from E")
+    _need((next_weight is None) == (next_out is None), "rmsnorm_add: the second norm needs its gain and its output")
+    if next_out is not None:
+        _need(next_weight.numel() == E and next_weight.is_contiguous() and next_out.is_contiguous()
+              and tuple(next_out.shape) == (R, E), "rmsnorm_add: the second norm's operands differ from [R, E]")
+    nb = R * E * 12 + _nbytes(weight, next_weight) + (0 if next_out is None else _nbytes(next_out))
+    with _timed("rmsnorm_add", nb, 8 * R * E, "fp32"):
+        _check(_lib().da_rmsnorm_add(_ptr(src), _ptr(weight), _dt(weight), _ptr(x), _ptr(next_weight),
+                                     _dt(next_weight) if next_weight is not None else 0, float(gain_offset), float(eps),
+                                     _ptr(next_out), _dt(next_out) if next_out is not None else 0, R, E, _stream()))
+
+
+def gated_act(gu: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
+    """mid[r, j] = act(gu[r, j]) * gu[r, inner + j]: the halves of a fused gate | up product."""
+    _dev(gu, mid)
+    _rows_2d(gu, "gu"); _rows_2d(mid, "mid")
+    R, inner = mid.shape
+    _need(gu.shape[0] == R and gu.shape[1] == 2 * inner and gu.dtype == mid.dtype, "gated_act: gu must be [R, 2 * inner] of mid's dtype")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"gated_act: unknown activation {act!r}")
+    with _timed("gated_act", _nbytes(gu, mid), 10 * R * inner, "fp32"):
+        _check(_lib().da_gated_act(_ptr(gu), gu.stride(0), _dt(gu), _ptr(mid), mid.stride(0), R, inner, ACTIVATIONS[act],
+                                   _stream()))
+    return mid
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "softcap: contiguous float32 logits")
+    _check(_lib().da_softcap(_ptr(logits), logits.numel(), float(cap), _stream()))
+    return logits
+
+
+# ------------------------------------------------------------------------------- experts
+MOE_TILE_ROWS = 64       # rows of a tile of the plain grouped products
+
+
+def moe_slot_space(n_tokens: int, top: int, n_experts: int, tile: int):
+    """(tiles, rows) of the slot space that holds every (token, choice) pair with each expert's pairs starting
+    at a multiple of ``tile`` rows, whatever the routing."""
+    tiles = -(-n_tokens * top // tile) + n_experts
+    return tiles, tiles * tile
+
+
+def moe_route(tokens: Optional[torch.Tensor], table: Optional[torch.Tensor], ids: Optional[torch.Tensor], n_tokens: int,
+              top: int, n_experts: int, tile: int, slot_of_pair: torch.Tensor, row_of_slot: torch.Tensor,
+              tile_expert: torch.Tensor) -> None:
+    """Every (token, choice) pair gets a slot; an expert's slots lie together and start at a multiple of ``tile``.
+    The experts come from ``table[tokens[n], k]`` or from ``ids[n, k]``."""
+    _dev(tokens, table, ids, slot_of_pair, row_of_slot, tile_expert)
+    for t_ in (tokens, table, ids, slot_of_pair, row_of_slot, tile_expert):
+        _need(t_ is None or (t_.dtype == torch.int32 and t_.is_contiguous()), "moe_route: int32 contiguous operands")
+    vocab = 0
+    if table is not None:
+        _need(tokens is not None and tokens.numel() >= n_tokens and table.dim() == 2 and table.shape[1] == top,
+              "moe_route: a table [vocab, top] with a token id a row")
+        vocab = table.shape[0]
+    else:
+        _need(ids is not None and ids.numel() >= n_tokens * top, "moe_route: expert ids [N, top]")
+    tiles, rows = moe_slot_space(n_tokens, top, n_experts, tile)
+    _need(slot_of_pair.numel() >= n_tokens * top and row_of_slot.numel() >= rows and tile_expert.numel() >= tiles,
+          "moe_route: the outputs are smaller than the slot space")
+    with _timed("moe_route", 4 * (n_tokens * top * 3 + rows + tiles), 0, "fp32"):
+        _check(_lib().da_moe_route(_ptr(tokens), _ptr(table), vocab, _ptr(ids), n_tokens, top, n_experts, tile,
+                                   _ptr(slot_of_pair), _ptr(row_of_slot), _ptr(tile_expert), rows, tiles, _stream()))
+
+
+def _moe_common(a, row_of_slot, tile_expert, w, tiles, tile, name):
+    _dev(a, row_of_slot, tile_expert, w)
+    _rows_2d(a, "a")
+    _need(w.dim() == 3 and w.is_contiguous() and w.dtype == a.dtype, f"{name}: stacked weights [experts, out, in] of a's dtype")
+    _need(row_of_slot.dtype == torch.int32 and tile_expert.dtype == torch.int32 and tile_expert.numel() >= tiles
+          and row_of_slot.numel() >= tiles * tile, f"{name}: the routing arrays are smaller than the slot space")
+
+
+def moe_gated_ref(a: torch.Tensor, row_of_slot: torch.Tensor, tile_expert: torch.Tensor, w: torch.Tensor,
+                  mid: torch.Tensor, tiles: int, act: str) -> torch.Tensor:
+    """mid[slot] = act(Wg_e a[row_of_slot[slot]]) * (Wu_e a[...]) for every used slot; w: [experts, 2 F, K]."""
+    _moe_common(a, row_of_slot, tile_expert, w, tiles, MOE_TILE_ROWS, "moe_gated")
+    K, F = a.shape[1], w.shape[1] // 2
+    _rows_2d(mid, "mid")
+    _need(w.shape[2] == K and w.shape[1] == 2 * F and mid.shape[1] == F and mid.shape[0] >= tiles * MOE_TILE_ROWS
+          and mid.dtype == a.dtype, "moe_gated: shapes differ")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"moe_gated: unknown activation {act!r}")
+    with _timed("moe_gated_plain", _nbytes(a, w, mid), 4 * tiles * MOE_TILE_ROWS * F * K, "fp32" if a.dtype == torch.float32 else "bf16"):
+        _check(_lib().da_moe_gated_ref(_ptr(a), a.stride(0), _dt(a), _ptr(row_of_slot), _ptr(tile_expert), _ptr(w),
+                                       _ptr(mid), mid.stride(0), tiles, K, F, ACTIVATIONS[act], _stream()))
+    return mid
+
+
+def moe_down_ref(mid: torch.Tensor, row_of_slot: torch.Tensor, tile_expert: torch.Tensor, w: torch.Tensor,
+                 out: torch.Tensor, tiles: int) -> torch.Tensor:
+    """out[slot] = Wd_e mid[slot] (32-bit) for every used slot; w: [experts, width, F]."""
+    _moe_common(mid, row_of_slot, tile_expert, w, tiles, MOE_TILE_ROWS, "moe_down")
+    F, width = mid.shape[1], w.shape[1]
+    _rows_2d(out, "out")
+    _need(w.shape[2] == F and out.shape[1] == width and out.dtype == torch.float32 and
+          out.shape[0] >= tiles * MOE_TILE_ROWS and mid.shape[0] >= tiles * MOE_TILE_ROWS, "moe_down: shapes differ")
+    with _timed("moe_down_plain", _nbytes(mid, w, out), 2 * tiles * MOE_TILE_ROWS * F * width, "fp32" if mid.dtype == torch.float32 else "bf16"):
+        _check(_lib().da_moe_down_ref(_ptr(mid), mid.stride(0), _dt(mid), _ptr(row_of_slot), _ptr(tile_expert), _ptr(w),
+                                      _ptr(out), out.stride(0), tiles, F, width, _stream()))
+    return out
+
+
+def moe_combine(out: torch.Tensor, slot_of_pair: torch.Tensor, weights: Optional[torch.Tensor], uniform: float,
+                top: int, y: torch.Tensor, accumulate: bool) -> torch.Tensor:
+    """y[n] (+)= sum_k weight * out[slot_of_pair[n, k]] with ``weights[n, k]`` or the one weight ``uniform``."""
+    _dev(out, slot_of_pair, weights, y)
+    _rows_2d(out, "out"); _rows_2d(y, "y")
+    N, width = y.shape
+    _need(out.dtype == torch.float32 and y.dtype == torch.float32 and out.shape[1] == width, "moe_combine: float32 [.., width]")
+    _need(slot_of_pair.dtype == torch.int32 and slot_of_pair.numel() >= N * top, "moe_combine: a slot a pair")
+    _need(weights is None or (weights.dtype == torch.float32 and weights.numel() >= N * top), "moe_combine: a weight a pair")
+    with _timed("moe_combine", (top + 2) * N * width * 4, top * N * width, "fp32"):
+        _check(_lib().da_moe_combine(_ptr(out), out.stride(0), _ptr(slot_of_pair), _ptr(weights), float(uniform), top,
+                                     _ptr(y), y.stride(0), N, width, int(accumulate), _stream()))
+    return y
+
+
 # ------------------------------------------------------------------------------- products
 def linear_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                act: Optional[str] = None, accumulate: bool = False) -> torch.Tensor:
@@ -323,6 +480,56 @@ def attention_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.
                               block_table.shape[1], _ptr(seq_of_token), _ptr(positions), N, n_heads, Hkv,
                               D, page, scale, int(window or 0), _ptr(out), out.stride(0),
                               _stream()))
+    return out
+
+
+def cache_page_elems(cache_slot: torch.Tensor) -> int:
+    return cache_slot[0].numel()
+
+
+def kv_write_split(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.Tensor, slot_map: torch.Tensor,
+                   n_kv_heads: int, head_dim: int, v_head_dim: int, page: int) -> None:
+    """Keys (``head_dim`` a head) and values (``v_head_dim`` a head) go to cache rows ``slot_map``; a page of the
+    slot holds Hkv * page * head_dim keys, then Hkv * v_head_dim * page values."""
+    _dev(qkv, cache_slot, slot_map)
+    _rows_2d(qkv, "qkv")
+    N = qkv.shape[0]
+    _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
+          "kv_write_split: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
+    _need(cache_slot.dtype == qkv.dtype, "kv_write_split: cache and activations differ in dtype")
+    _need(slot_map.dtype == torch.int32 and slot_map.numel() >= N, "kv_write_split: slot_map must be int32 [N]")
+    with _timed("kv_write", 2 * N * n_kv_heads * (head_dim + v_head_dim) * qkv.element_size(), 0, "fp32"):
+        _check(_lib().da_kv_write_split(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(cache_slot), _ptr(slot_map),
+                                        N, n_kv_heads, head_dim, v_head_dim, page, _stream()))
+
+
+def attention_rel_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
+                      positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, v_head_dim: int, page: int,
+                      scale: float, window: Optional[int], dist_bias: Optional[torch.Tensor], temp_coef: float,
+                      temp_every: int, out: torch.Tensor) -> torch.Tensor:
+    """Plain paged attention with a bias by distance (``dist_bias`` [Hq, n_dist] float32, the last column for every
+    larger distance), a query temperature by position, and values of their own size."""
+    _dev(q, cache_slot, block_table, seq_of_token, positions, dist_bias, out)
+    _rows_2d(q, "q"); _rows_2d(out, "out")
+    N = q.shape[0]
+    _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
+          "attention: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
+    _need(q.shape[1] == n_heads * head_dim and out.shape[1] == n_heads * v_head_dim and out.shape[0] == N,
+          "attention: q must be [N, Hq*D] and out [N, Hq*Dv]")
+    _need(q.dtype == cache_slot.dtype == out.dtype, "attention: q, cache and out must share a dtype")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "attention: block_table must be contiguous int32 [S, max_blocks]")
+    _need(seq_of_token.dtype == torch.int32 and positions.dtype == torch.int32, "attention: ids must be int32")
+    _need(seq_of_token.numel() >= N and positions.numel() >= N, "attention: fewer ids than rows")
+    n_dist = 0
+    if dist_bias is not None:
+        _need(dist_bias.dtype == torch.float32 and dist_bias.is_contiguous() and dist_bias.dim() == 2
+              and dist_bias.shape[0] == n_heads, "attention: the bias by distance must be float32 [Hq, n_dist]")
+        n_dist = dist_bias.shape[1]
+    _check(_lib().da_attn_rel_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table), block_table.shape[1],
+                                  _ptr(seq_of_token), _ptr(positions), N, n_heads, n_kv_heads, head_dim, v_head_dim, page,
+                                  float(scale), int(window or 0), _ptr(dist_bias), n_dist, float(temp_coef),
+                                  int(temp_every), _ptr(out), out.stride(0), _stream()))
     return out
 
 
@@ -646,3 +853,42 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
         return out
     with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, scale, window, out)
+
+
+def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, n_kv_heads: int,
+                        head_dim: int, v_head_dim: int, scale: float, window: Optional[int],
+                        dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
+                        out: torch.Tensor) -> torch.Tensor:
+    """Attention of every row of the step with a bias by distance, a query temperature and values of their own
+    size (each optional).  32-bit, the reference mode and shapes the matrix-core kernels do not take use the
+    plain kernel for all rows."""
+    bt = ctx.block_tables[group]
+    page = ctx.cache.page_size
+    with _timed("attention_plain", 0, 0, "fp32" if q.dtype == torch.float32 else "bf16"):
+        return attention_rel_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, n_kv_heads, head_dim,
+                                 v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out)
+
+
+def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
+    """mid = act(h @ gate.T) * (h @ up.T) with gate | up as one matrix [2 inner, width]."""
+    N, inner = mid.shape
+    gu = ctx.buf("ff_gate_up", N, 2 * inner, h.dtype)
+    linear(h, gate_up, None, gu)
+    return gated_act(gu, mid, act)
+
+
+def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                    n_experts: int, top: int, weight: float, act: str, x: torch.Tensor, accumulate: bool) -> torch.Tensor:
+    """x (+)= sum_k weight * expert_{table[token, k]}(h): route, two grouped products, combine."""
+    N, width = h.shape
+    inner = down.shape[2]
+    tile = MOE_TILE_ROWS
+    tiles, rows = moe_slot_space(N, top, n_experts, tile)
+    ints = ctx.buf("moe_route", N * top + rows + tiles, 1, torch.int32).view(-1)
+    slot_of_pair, row_of_slot, tile_expert = ints[:N * top], ints[N * top:N * top + rows], ints[N * top + rows:]
+    moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
+    mid = ctx.buf("moe_mid", rows, inner, h.dtype)
+    pair_out = ctx.buf("moe_out", rows, width, torch.float32)
+    moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
+    moe_down_ref(mid, row_of_slot, tile_expert, down, pair_out, tiles)
+    return moe_combine(pair_out, slot_of_pair, None, weight, top, x, accumulate)

@@ -1,4 +1,5 @@
 from . import gpt2  # noqa: F401  (registers GPT2LMHeadModel)
+from . import virudra  # noqa: F401  (registers Virudra)
 from .causal_lm import CausalLM, load_model
 
 __all__ = ["CausalLM", "load_model"]

@@ -104,6 +104,8 @@ class CausalLM:
             ops.linear(e, self.head_weight, None, logits)
         if self.config.logit_multiplier != 1.0:     # (an architecture's constant; GPT-2 has none)
             ops.copy_rows(logits, logits, scale=1.0 / self.config.logit_multiplier)
+        if self.config.logit_softcap > 0.0:         # logits <- cap * tanh(logits / cap)
+            ops.softcap(logits, self.config.logit_softcap)
         return logits
 
 

@@ -3,11 +3,18 @@
 Fused projection to q | k | v (+ bias), optional position encoding of q and k, write of the
 new k and v rows into the cache slot, attention of every row over its sequence's pages, and
 the output projection (+ bias) added into the residual stream.
+
+Optional extras, each a record of the spec with its constants: values of a per-head size of their own
+(``v_head_dim``), a learned bias by the distance between query and key (``distance_bias``, a table of
+buckets that the mixer writes out once as a table by distance), and a query temperature that grows with
+the position (``query_temperature``).  Positions enter such a mixer through these only.
 Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:226-420
 (projections :266-291, cache write :315-336, scores/softmax/weighted sum :458-532, output
 projection :385-408); the residual add is TransformerBlock.java:176.
 """
 from __future__ import annotations
+
+import math
 
 import torch
 
@@ -15,8 +22,28 @@ from ..kernels import ops
 from .base import (KVNeed, Mixer, StepContext, build_position, register_mixer, to_matrix, to_vector)
 
 
+def distance_bucket(n: int, n_buckets: int, max_distance: int) -> int:
+    """The row of a bias table of ``n_buckets`` rows that the distance ``n`` >= 0 uses: one row a distance below
+    half the rows, then rows shared in steps that grow like a logarithm up to ``max_distance``."""
+    half = n_buckets // 2
+    if n < half:
+        return n
+    return min(n_buckets - 1, half + int(math.floor(math.log(n / half) / math.log(max_distance / half) * (n_buckets - half))))
+
+
+def bias_by_distance(table: torch.Tensor, max_distance: int) -> torch.Tensor:
+    """A bucket table [n_buckets, heads] written out by distance: float32 [heads, max_distance + 1] on the CPU;
+    every distance from ``max_distance`` on uses the last column (it lies in the last bucket)."""
+    n_buckets = table.shape[0]
+    if n_buckets < 2 or max_distance <= n_buckets // 2:
+        raise ValueError(f"a bias table of {n_buckets} rows with a largest distance of {max_distance}")
+    rows = torch.tensor([distance_bucket(n, n_buckets, max_distance) for n in range(max_distance + 1)], dtype=torch.long)
+    return table.detach().to("cpu", torch.float32)[rows].t().contiguous()
+
+
 class CausalSelfAttention(Mixer):
     graph_safe = True
+    can_store = True          # with ``ctx.part_accumulate`` off the output projection stores instead of adding
 
     def __init__(self, spec, params, dtype, device):
         self.spec = spec
@@ -27,9 +54,14 @@ class CausalSelfAttention(Mixer):
         # the others (and everything in 32-bit) on the plain attention kernel.
         if not (1 <= self.head_dim <= ops.MAX_HEAD_DIM):
             raise ValueError(f"head size {self.head_dim} is outside 1..{ops.MAX_HEAD_DIM}")
+        self.v_head_dim = int(getattr(spec, "v_head_dim", None) or self.head_dim)
+        if not (1 <= self.v_head_dim <= ops.MAX_HEAD_DIM):
+            raise ValueError(f"value head size {self.v_head_dim} is outside 1..{ops.MAX_HEAD_DIM}")
         self.q_cols = self.n_heads * self.head_dim
         self.kv_cols = self.n_kv_heads * self.head_dim
-        self.qkv_cols = self.q_cols + 2 * self.kv_cols
+        self.v_cols = self.n_kv_heads * self.v_head_dim
+        self.o_cols = self.n_heads * self.v_head_dim
+        self.qkv_cols = self.q_cols + self.kv_cols + self.v_cols
         self.scale = float(spec.scale)
         self.window = spec.window
         self.qkv_weight = to_matrix(params["qkv_weight"], dtype, device)
@@ -38,20 +70,40 @@ class CausalSelfAttention(Mixer):
         self.out_bias = to_vector(params.get("out_bias"), dtype, device) if spec.out_bias else None
         if tuple(self.qkv_weight.shape) != (self.qkv_cols, spec.width):
             raise ValueError(f"qkv weight is {list(self.qkv_weight.shape)}, expected {[self.qkv_cols, spec.width]}")
-        if tuple(self.out_weight.shape) != (spec.width, self.q_cols):
-            raise ValueError(f"output weight is {list(self.out_weight.shape)}, expected {[spec.width, self.q_cols]}")
+        if tuple(self.out_weight.shape) != (spec.width, self.o_cols):
+            raise ValueError(f"output weight is {list(self.out_weight.shape)}, expected {[spec.width, self.o_cols]}")
+        # the extras: a table by distance [heads, max_distance + 1] (32-bit) and the temperature's constants
+        self.dist_bias = None
+        db = getattr(spec, "distance_bias", None)
+        if db is not None:
+            table = params["distance_bias"]
+            if table.dim() != 2 or table.shape[1] != self.n_heads or (db.n_buckets and table.shape[0] != db.n_buckets):
+                raise ValueError(f"distance-bias table is {list(table.shape)}, expected "
+                                 f"{[db.n_buckets or 'rows', self.n_heads]}")
+            self.dist_bias = bias_by_distance(table, db.max_distance).to(device)
+        qt = getattr(spec, "query_temperature", None)
+        self.temp_coef, self.temp_every = (float(qt.coef), int(qt.every)) if qt is not None else (0.0, 0)
+        if qt is not None and self.temp_every <= 0:
+            raise ValueError(f"query temperature period {self.temp_every} must be positive")
+        self.extras = self.dist_bias is not None or self.temp_every > 0 or self.v_head_dim != self.head_dim
         self.position = None
         if spec.position is not None and spec.position.kind != "none":
             self.position = build_position(spec.position, params.get("position", {}), dtype, device)
 
     def cache_need(self):
-        return KVNeed(self.n_kv_heads, self.head_dim, self.window)
+        return KVNeed(self.n_kv_heads, self.head_dim, self.window,
+                      None if self.v_head_dim == self.head_dim else self.v_head_dim)
+
+    def _epilogue_write(self) -> bool:
+        """Whether the q|k|v product may write keys and values to the cache itself (its epilogue assumes
+        keys and values of one size)."""
+        return self.position is None and self.v_head_dim == self.head_dim
 
     def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call) -> bool:
         """Small steps: LayerNorm, the q|k|v projection and the cache write in one kernel."""
         N = x.shape[0]
         ln = norm.fusable_params()
-        if ln is None or self.position is not None or not ops.can_fuse_ln(N, x, self.qkv_weight):
+        if ln is None or not self._epilogue_write() or not ops.can_fuse_ln(N, x, self.qkv_weight):
             return False
         gain, bias, eps = ln
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
@@ -68,7 +120,7 @@ class CausalSelfAttention(Mixer):
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
-        if self.position is None and call.write:
+        if self._epilogue_write() and call.write:
             # the new keys and values go to the cache in the projection's epilogue
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv, kv_cache=slot, slot_map=ctx.slot_maps[group],
                        q_cols=self.q_cols)
@@ -76,16 +128,24 @@ class CausalSelfAttention(Mixer):
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
             if self.position is not None:
                 self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
-            if call.write:
+            if call.write and self.v_head_dim == self.head_dim:
                 ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
                              self.n_kv_heads, self.head_dim)
+            elif call.write:
+                ops.kv_write_split(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
+                                   self.n_kv_heads, self.head_dim, self.v_head_dim, ctx.cache.page_size)
         self._attend(ctx, qkv, x, slot, group, call)
 
     def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int,
                 call) -> None:
         N = qkv.shape[0]
-        o = ctx.buf("attn_out", N, self.q_cols, ctx.dtype)
-        ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
+        o = ctx.buf("attn_out", N, self.o_cols, ctx.dtype)
+        if self.extras:
+            ops.paged_attention_rel(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.n_kv_heads, self.head_dim,
+                                    self.v_head_dim, self.scale, self.window, self.dist_bias, self.temp_coef,
+                                    self.temp_every, o)
+        else:
+            ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
         if ctx.debug_hook is not None:      # the reference's stage names (CausalSelfAttention.java:299-301,384)
             ctx.emit(call.layer, "query_projection", qkv[:, :self.q_cols])
             ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
@@ -94,7 +154,7 @@ class CausalSelfAttention(Mixer):
             # the output projection before its bias (CausalSelfAttention.java:406), worked out once more for the hook
             ctx.emit(call.layer, "attention_output",
                      ops.linear(o, self.out_weight, None, ctx.buf("attn_proj_debug", N, x.shape[1], torch.float32)))
-        ops.linear(o, self.out_weight, self.out_bias, x, accumulate=True)
+        ops.linear(o, self.out_weight, self.out_bias, x, accumulate=ctx.part_accumulate)
 
 
 register_mixer("attention", CausalSelfAttention)

@@ -35,9 +35,11 @@ import torch
 
 @dataclass(frozen=True)
 class KVNeed:
+    """Pages of keys (``head_dim`` a head) and values (``v_head_dim`` a head; None: the keys' size)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -96,6 +98,9 @@ class StepContext:
         self.slot_maps: List[torch.Tensor] = []        # per group int32 [N]
         self.cache = None                              # engine.DeviceCache
         self._arena = None
+        # False while a part runs that was given a buffer of its own to fill (a norm follows it): a part
+        # with ``can_store`` then stores its result there instead of adding to what the buffer holds
+        self.part_accumulate = True
         # Called as hook(layer, stage, tensor) with copies of named intermediates (layer -1: the
         # embedding), when set: core/src/main/java/io/teknek/deliverance/model/AbstractModel.java:122-128,505-515.
         self.debug_hook: Optional[Callable] = None

@@ -34,36 +34,55 @@ class Block:
         h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)      # no norm in front: the stream, converted
         return ops.copy_rows(x, h)
 
-    def _part(self, ctx, x, pre, post, run, run_normed):
+    def _part(self, ctx, x, pre, post, run, run_normed, part=None, h_ready=None, next_pre=None):
         """One part of the block.  Parts add into the tensor they are given.  Without a norm behind
-        the part (and without a multiplier) that tensor is the residual stream; else the part adds
-        into a buffer of its own (cleared by a fill kernel of the engine's, so that a recorded step
-        holds no memset), whose norm, kept in 32-bit, times the multiplier is then added to the stream."""
+        the part (and without a multiplier) that tensor is the residual stream; else the part gets
+        a buffer of its own (cleared by a fill kernel of the engine's, so that a recorded step
+        holds no memset; a part with ``can_store`` stores into it instead and nothing is cleared), whose
+        norm, kept in 32-bit, times the multiplier is then added to the stream.  ``h_ready``: the part's
+        normalised input, when the norm behind the part before has already made it.  Returns the
+        normalised input of the part that follows (``next_pre`` of the new stream) when the norm behind
+        this part could make it in the same pass (``Norm.add_into``), else None."""
         target = x
         own = post is not None or self.residual_multiplier != 1.0
+        stores = own and getattr(part, "can_store", False)
         if own:
-            target = ops.fill_zero(ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32))
-        # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
-        # of it itself (fused into its first product) and returns True, or returns False to
-        # decline this step.  That needs the part's input and the tensor it adds into to be the same.
-        if not (not own and pre is not None and run_normed is not None and run_normed(pre)):
-            run(Block._normed(ctx, x, pre), target)
+            target = ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32)
+            if not stores:
+                ops.fill_zero(target)
+        ctx.part_accumulate = not stores
+        try:
+            # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
+            # of it itself (fused into its first product) and returns True, or returns False to
+            # decline this step.  That needs the part's input and the tensor it adds into to be the same.
+            if h_ready is not None:
+                run(h_ready, target)
+            elif not (not own and pre is not None and run_normed is not None and run_normed(pre)):
+                run(Block._normed(ctx, x, pre), target)
+        finally:
+            ctx.part_accumulate = True
         if own:
+            add_into = None if post is None or self.residual_multiplier != 1.0 else getattr(post, "add_into", None)
+            if add_into is not None:         # norm, addition and the next part's norm in one pass over the rows
+                return add_into(ctx, target, x, next_pre, next_name="norm_ahead")
             out = target if post is None else post.forward(ctx, target, out_name="post_norm", out_dtype=torch.float32)
             ops.copy_rows(out, x, accumulate=True, scale=self.residual_multiplier)
+        return None
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
         fused = getattr(self.mixer, "forward_normed", None)
-        self._part(ctx, x, self.pre_mixer_norm, self.post_mixer_norm,
-                   lambda h, into: self.mixer.forward(ctx, h, into, call),
-                   None if fused is None else (lambda norm: fused(ctx, norm, x, call)))
+        h_ff = self._part(ctx, x, self.pre_mixer_norm, self.post_mixer_norm,
+                          lambda h, into: self.mixer.forward(ctx, h, into, call),
+                          None if fused is None else (lambda norm: fused(ctx, norm, x, call)), part=self.mixer,
+                          next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else self.pre_ff_norm)
         if ctx.debug_hook is not None:
             ctx.emit(call.layer, "post_attention_residual", x)
         if self.feed_forward is not None:
             fused = getattr(self.feed_forward, "forward_normed", None)
             self._part(ctx, x, self.pre_ff_norm, self.post_ff_norm,
                        lambda h, into: self.feed_forward.forward(ctx, h, into),
-                       None if fused is None else (lambda norm: fused(ctx, norm, x)))
+                       None if fused is None else (lambda norm: fused(ctx, norm, x)), part=self.feed_forward,
+                       h_ready=h_ff)
             if ctx.debug_hook is not None:
                 ctx.emit(call.layer, "post_ff_residual", x)
         if self.post_block_norm is not None:                # the stream itself, normalised in place

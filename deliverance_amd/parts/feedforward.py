@@ -45,3 +45,70 @@ class DenseFeedForward(FeedForward):
 
 
 register_feed_forward("dense", DenseFeedForward)
+
+
+class GatedFeedForward(FeedForward):
+    """``down(act(gate h) * (up h))`` without biases; gate and up are one matrix [2 inner, width] (gate rows
+    first), so one product reads h once."""
+    graph_safe = True
+    can_store = True
+
+    def __init__(self, spec, params, dtype, device):
+        self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {self.activation!r}")
+        self.gate_up_weight = to_matrix(params["gate_up_weight"], dtype, device)
+        self.down_weight = to_matrix(params["down_weight"], dtype, device)
+        if tuple(self.gate_up_weight.shape) != (2 * self.inner, self.width):
+            raise ValueError(f"gate|up weight is {list(self.gate_up_weight.shape)}, expected {[2 * self.inner, self.width]}")
+        if tuple(self.down_weight.shape) != (self.width, self.inner):
+            raise ValueError(f"down weight is {list(self.down_weight.shape)}, expected {[self.width, self.inner]}")
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
+        N = h.shape[0]
+        mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)
+        ops.gated_linear(ctx, h, self.gate_up_weight, mid, self.activation)
+        ops.linear(mid, self.down_weight, None, x, accumulate=ctx.part_accumulate)
+
+
+class ExpertsFeedForward(FeedForward):
+    """A mixture of gated experts.  The router says which ``top`` experts a token uses and with what weights;
+    ``token_table``: row ``token id`` of an integer table names them, each with weight 1 / top.  The step's
+    (token, choice) pairs are laid out expert by expert on the device (``ops.moe_route``), two grouped
+    products run over that layout, and the pairs' results are added up per token.  Nothing is read back to the
+    host, so a step can be recorded."""
+    graph_safe = True
+    can_store = True
+
+    def __init__(self, spec, params, dtype, device):
+        self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
+        self.n_experts, self.top, self.router = spec.n_experts, spec.top, spec.router
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {self.activation!r}")
+        if self.router != "token_table":
+            raise ValueError(f"unknown router {self.router!r}; known: 'token_table'")
+        if not (1 <= self.top <= self.n_experts):
+            raise ValueError(f"top {self.top} of {self.n_experts} experts")
+        self.gate_up_weight = to_matrix(params["gate_up_weight"], dtype, device)       # [experts, 2 inner, width]
+        self.down_weight = to_matrix(params["down_weight"], dtype, device)             # [experts, width, inner]
+        if tuple(self.gate_up_weight.shape) != (self.n_experts, 2 * self.inner, self.width):
+            raise ValueError(f"experts' gate|up weights are {list(self.gate_up_weight.shape)}, expected "
+                             f"{[self.n_experts, 2 * self.inner, self.width]}")
+        if tuple(self.down_weight.shape) != (self.n_experts, self.width, self.inner):
+            raise ValueError(f"experts' down weights are {list(self.down_weight.shape)}, expected "
+                             f"{[self.n_experts, self.width, self.inner]}")
+        table = params["table"]
+        if table.dim() != 2 or table.shape[1] != self.top or (spec.vocab_size and table.shape[0] != spec.vocab_size):
+            raise ValueError(f"expert table is {list(table.shape)}, expected {[spec.vocab_size or 'vocab', self.top]}")
+        if table.dtype not in (torch.int32, torch.int64) or int(table.min()) < 0 or int(table.max()) >= self.n_experts:
+            raise ValueError(f"expert table must hold integers in 0..{self.n_experts - 1}")
+        self.table = table.to(device=device, dtype=torch.int32).contiguous()
+        self.weight = 1.0 / self.top
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
+        ops.experts_forward(ctx, h, self.table, self.gate_up_weight, self.down_weight, self.n_experts, self.top,
+                            self.weight, self.activation, x, accumulate=ctx.part_accumulate)
+
+
+register_feed_forward("gated", GatedFeedForward)
+register_feed_forward("experts", ExpertsFeedForward)

@@ -31,3 +31,44 @@ class LayerNorm(Norm):
 
 
 register_norm("layernorm", LayerNorm)
+
+
+class RmsNorm(Norm):
+    """The row divided by its root mean square (eps inside the root), times ``gain_offset + weight``; all in
+    32-bit.  Behind a part it can do three things in one pass over the row (``add_into``): normalise the
+    part's output, add it to the residual stream, and normalise the new stream for the part that follows."""
+
+    def __init__(self, spec, params, dtype, device):
+        self.width = spec.width
+        self.eps = float(spec.eps)
+        self.gain_offset = float(getattr(spec, "gain_offset", 0.0))
+        self.weight = to_vector(params["weight"], dtype, device)
+        if self.weight.numel() != self.width:
+            raise ValueError(f"RMS norm gain has {self.weight.numel()} entries for width {self.width}")
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                n_rows: Optional[int] = None, out_name: str = "norm",
+                out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        R = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        out = ctx.buf(out_name, R, self.width, out_dtype or ctx.dtype)
+        return ops.rmsnorm(x, self.weight, self.gain_offset, self.eps, out, rows)
+
+    def rms_params(self):
+        """(gain, gain_offset, eps): for kernels that apply this norm to their own rows."""
+        return self.weight, self.gain_offset, self.eps
+
+    def add_into(self, ctx: StepContext, src: torch.Tensor, x: torch.Tensor, next_norm=None,
+                 next_name: str = "norm") -> Optional[torch.Tensor]:
+        """x += norm(src).  With ``next_norm`` (an RMS norm of the same eps and offset) also returns
+        ``next_norm(x)`` of the new x in the compute dtype; returns None when it did not do that."""
+        nxt = next_norm if (type(next_norm) is RmsNorm and next_norm.eps == self.eps
+                            and next_norm.gain_offset == self.gain_offset and next_norm.width == self.width) else None
+        if nxt is None:
+            ops.rmsnorm_add(src, self.weight, x, self.gain_offset, self.eps)
+            return None
+        h = ctx.buf(next_name, x.shape[0], self.width, ctx.dtype)
+        ops.rmsnorm_add(src, self.weight, x, self.gain_offset, self.eps, nxt.weight, h)
+        return h
+
+
+register_norm("rmsnorm", RmsNorm)

@@ -60,7 +60,9 @@ class ModelSupport:
     @classmethod
     def detect(cls, config: dict) -> Architecture:
         """By ``architectures[0]``, else by ``model_type`` (ModelSupport.java:75-95)."""
-        archs = config.get("architectures") or []
+        archs = list(config.get("architectures") or [])
+        if isinstance(config.get("architecture"), str):      # some designs name one architecture, not a list
+            archs.append(config["architecture"])
         for n in archs:
             if isinstance(n, str) and n.lower() in cls._by_name:
                 return cls._by_name[n.lower()]

@@ -49,8 +49,10 @@ class WeightError(ValueError):
 @dataclass(frozen=True)
 class TensorDecl:
     name: str
-    shape: Tuple[int, ...]
-    init: str = "normal"         # "normal" | "ones_plus_normal" | "zeros" | "ones"
+    shape: Tuple[int, ...]       # a dimension of -1 is the checkpoint's to say
+    # "normal" | "ones_plus_normal" | "zeros" | "ones" | "distinct_ints" (int32 rows of different
+    # integers below ``std``: an expert table)
+    init: str = "normal"
     std: float = 0.02
     optional: bool = False       # absent is fine (e.g. an untied head falling back to the table)
 
@@ -89,7 +91,7 @@ def load_declared(folder: str, decls: Iterable[TensorDecl], ignore: Sequence[str
                 missing.append(d.name)
             continue
         dtype, shape = source.info(stored)
-        if tuple(shape) != tuple(d.shape):
+        if len(shape) != len(d.shape) or any(e != -1 and e != f for e, f in zip(d.shape, shape)):
             wrong_shape.append((d.name, d.shape, shape))
             continue
         t = source.tensor(stored)
@@ -117,6 +119,14 @@ def _generator_for(seed: int, name: str) -> torch.Generator:
 
 def draw_tensor(decl: TensorDecl, seed: int, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     g = _generator_for(seed, decl.name)
+    if any(n < 0 for n in decl.shape):
+        raise ValueError(f"tensor {decl.name}: a dimension that only a checkpoint names ({list(decl.shape)}) cannot be drawn")
+    if decl.init == "distinct_ints":
+        rows, top = decl.shape
+        n = int(decl.std)
+        if top > n:
+            raise ValueError(f"tensor {decl.name}: {top} different integers below {n}")
+        return torch.argsort(torch.rand((rows, n), generator=g), dim=1)[:, :top].to(torch.int32).contiguous()
     if decl.init == "zeros":
         t = torch.zeros(decl.shape, dtype=torch.float32)
     elif decl.init == "ones":

@@ -115,6 +115,12 @@ static inline int simt_update_dpp(int old, int src, int ctrl, int row_mask, int 
 static inline int simt_readlane(int v, int lane) { return (int)simt::lane_exchange((uint32_t)v, lane, 0u); }
 #define __builtin_amdgcn_readlane(v, l) simt_readlane((v), (l))
 #define __builtin_amdgcn_readfirstlane(v) simt_readlane((v), 0)
+// Fibers take turns and give way at barriers and lane exchanges only, so a read-modify-write is whole.
+static inline int atomicAdd(int* p, int v) {
+  const int old = *p;
+  *p = old + v;
+  return old;
+}
 static inline float __shfl_xor(float v, int mask, int) {
   return __uint_as_float(simt::lane_exchange(__float_as_uint(v), simt::lane_id() ^ mask, 0u));
 }
