@@ -16,9 +16,28 @@
 //
 // Formulas: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:504-532;
 // tensor/src/main/java/io/teknek/deliverance/tensor/operations/TensorOperations.java:240-272.
+//
+// Compiled a second time with DEC_REL (attn_decode_rel.hip) the kernel also takes what some designs put on the
+// scores: a bias by the distance between query and key (a table [Hq][n_dist], 32-bit, the last entry for every
+// larger distance) and a query temperature 1 + t_coef * ln(floor((p + 1) / t_every) + 1) that multiplies the
+// scale.  The plain build has none of that code.
 #include "common.h"
 
 #define DEC_MAX_D 256
+
+#ifdef DEC_REL
+#define DEC_KERNEL attn_decode_rel_kernel
+#define DEC_MERGE_KERNEL attn_decode_rel_merge_kernel
+#define DEC_REL_PARAMS , const float* __restrict__ rel_bias, int n_dist, float t_coef, int t_every
+#define DEC_REL_DECL , const float* rel_bias, int n_dist, float t_coef, int t_every
+#define DEC_REL_ARGS , rel_bias, n_dist, t_coef, t_every
+#else
+#define DEC_KERNEL attn_decode_kernel
+#define DEC_MERGE_KERNEL attn_decode_merge_kernel
+#define DEC_REL_PARAMS
+#define DEC_REL_DECL
+#define DEC_REL_ARGS
+#endif
 
 // e^x by the hardware's exp2 (two instructions; the library's expf is a dozen, and the merge of 16 wavefronts'
 // partial results takes 16 of them on the one wavefront that everything waits for)
@@ -35,10 +54,10 @@ __device__ __forceinline__ float dec_exp(float x) { return __builtin_amdgcn_exp2
 template <int CPR, int DEC_WAVES, bool SPLIT>
 // (registers are held to 128 for head sizes up to 64, so that two workgroups share a compute unit)
 __global__ void __launch_bounds__(DEC_WAVES * DA_WAVE, (CPR <= 8 || DEC_WAVES == 16) ? 4 : 2)
-attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
-                   const int* __restrict__ block_table, int max_blocks,
-                   const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
-                   int window, bf16_t* __restrict__ out, int out_ld, int span, float* __restrict__ partial) {
+DEC_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
+           const int* __restrict__ block_table, int max_blocks,
+           const int* __restrict__ seq_lens, int Hq, int Hkv, int D, int page, float scale,
+           int window, bf16_t* __restrict__ out, int out_ld, int span, float* __restrict__ partial DEC_REL_PARAMS) {
   constexpr int G = DA_WAVE / CPR;            // keys scored side by side
   constexpr int DPL = CPR <= 8 ? 1 : CPR / 8; // value dimensions per lane: D <= 8 * CPR <= 64 * DPL
   __shared__ __attribute__((aligned(16))) float ps[DEC_WAVES][DA_WAVE];
@@ -84,6 +103,12 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
   const int p = SPLIT ? (p_row < split0 + span - 1 ? p_row : split0 + span - 1) : p_row;
   const int lo = SPLIT ? (lo_row > split0 ? lo_row : split0) : lo_row;
+#ifdef DEC_REL
+  const float* brow = rel_bias ? rel_bias + (size_t)h * n_dist : nullptr;
+  const float qscale = t_every > 0 ? scale * (1.0f + t_coef * logf((float)((p_row + 1) / t_every + 1))) : scale;
+#else
+  const float qscale = scale;
+#endif
 
   float acc[DPL];
 #pragma unroll
@@ -163,6 +188,15 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
         vv0[g] = *(const uint4*)(vbase + pg * page_elems + d * page + (gs & pmask));
       }
     }
+#ifdef DEC_REL
+    // the bias of the key whose score this lane will keep, asked for beside the keys and values (a key past the
+    // row's own position has no distance: it reads entry 0 and is dropped with its score)
+    float brel = 0.f;
+    if (brow) {
+      const int dist = p_row - (c0 + piece * G + sub);
+      brel = brow[dist < 0 ? 0 : (dist < n_dist ? dist : n_dist - 1)];
+    }
+#endif
     // nothing moves across this line: the compiler would otherwise push the value loads down behind
     // the scores to save registers, and a chunk would cost a third memory round trip
     __builtin_amdgcn_sched_barrier(0);
@@ -171,8 +205,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
       const uint32_t u[4] = {qraw.x, qraw.y, qraw.z, qraw.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        qf[2 * e] = piece_ok ? __uint_as_float(u[e] << 16) * scale : 0.f;
-        qf[2 * e + 1] = piece_ok ? __uint_as_float(u[e] & 0xffff0000u) * scale : 0.f;
+        qf[2 * e] = piece_ok ? __uint_as_float(u[e] << 16) * qscale : 0.f;
+        qf[2 * e + 1] = piece_ok ? __uint_as_float(u[e] & 0xffff0000u) * qscale : 0.f;
       }
     }
 #pragma unroll
@@ -193,6 +227,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     const int kidx = piece * G + sub;                 // which key of the chunk this lane kept
     const int key = c0 + kidx;
     const bool valid = key >= lo && key <= p;
+#ifdef DEC_REL
+    mine += brel;                                     // (-inf stays -inf)
+#endif
     const float m_new = fmaxf(m, wave_max(mine));
     const float e = valid ? dec_exp(mine - m_new) : 0.f;
     const float alpha = dec_exp(m - m_new);
@@ -298,7 +335,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
 
 // The partial results of a (sequence, head) pair, merged in ascending order of the shares.
 __global__ void __launch_bounds__(256)
-attn_decode_merge_kernel(const float* __restrict__ partial, int n_splits, int Hq, int D,
+DEC_MERGE_KERNEL(const float* __restrict__ partial, int n_splits, int Hq, int D,
                          bf16_t* __restrict__ out, int out_ld) {
   const int s = blockIdx.x / Hq, h = blockIdx.x % Hq;
   const float* mine = partial + (size_t)blockIdx.x * n_splits * (D + 2);
@@ -338,16 +375,16 @@ static int decode_checks(const void* q, int q_ld, const void* cache, int max_blo
 // (S * Hq * n_splits * (D + 2) floats), then the merge kernel.
 static int decode_launch(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
                          const int* seq_lens, int S, int Hq, int Hkv, int D, int page, float scale, int window,
-                         void* out, int out_ld, int n_splits, int span, float* partial, hipStream_t st) {
+                         void* out, int out_ld, int n_splits, int span, float* partial, hipStream_t st DEC_REL_DECL) {
   const int pieces = D / 8;
   // 8 wavefronts; 16 where the workgroups are no more than the compute units (a context above 512 is then
   // still one chunk a wavefront, and the larger workgroup's start is paid once per compute unit)
   const bool wide = (long)S * Hq * n_splits <= 256 && pieces <= 8;     // larger heads need the registers of 8 wavefronts
   dim3 grid(S * Hq, n_splits);
 #define LAUNCH3(C, W, SP)                                                                                   \
-  hipLaunchKernelGGL((attn_decode_kernel<C, W, SP>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, \
+  hipLaunchKernelGGL((DEC_KERNEL<C, W, SP>), grid, dim3(W * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, \
                      (const bf16_t*)cache, block_table, max_blocks, seq_lens, Hq, Hkv, D, page, scale, window, \
-                     (bf16_t*)out, out_ld, span, partial)
+                     (bf16_t*)out, out_ld, span, partial DEC_REL_ARGS)
 #define LAUNCH2(C, W) do { if (n_splits > 1) LAUNCH3(C, W, true); else LAUNCH3(C, W, false); } while (0)
 #define LAUNCH(C) do { if (wide) LAUNCH2(C, 16); else LAUNCH2(C, 8); } while (0)
   if (pieces <= 2) LAUNCH(2);
@@ -359,11 +396,43 @@ static int decode_launch(const void* q, int q_ld, const void* cache, const int* 
 #undef LAUNCH2
 #undef LAUNCH3
   if (n_splits > 1)
-    hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(S * Hq), dim3(D <= 64 ? 64 : (D <= 128 ? 128 : 256)), 0, st,
+    hipLaunchKernelGGL(DEC_MERGE_KERNEL, dim3(S * Hq), dim3(D <= 64 ? 64 : (D <= 128 ? 128 : 256)), 0, st,
                        partial, n_splits, Hq, D, (bf16_t*)out, out_ld);
   return 0;
 }
 
+#ifdef DEC_REL
+static int rel_checks(const float* rel_bias, int n_dist, int t_every) {
+  DA_REQUIRE(!rel_bias || n_dist > 0, "attn_decode_rel: a bias table without entries");
+  DA_REQUIRE(t_every >= 0, "attn_decode_rel: bad temperature period %d", t_every);
+  return 0;
+}
+
+// n_splits <= 1: one workgroup a (sequence, head) pair; else the keys of a pair go to n_splits workgroups
+// and `workspace` holds the partial results.
+extern "C" int da_attn_decode_rel(const void* q, int q_ld, const void* cache, const int* block_table,
+                                  int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
+                                  float scale, int window, const float* rel_bias, int n_dist, float t_coef,
+                                  int t_every, void* out, int out_ld, int n_splits, void* workspace,
+                                  long workspace_bytes, void* stream) {
+  if (decode_checks(q, q_ld, cache, max_blocks, S, Hq, Hkv, D, page, window, out_ld)) return 1;
+  if (rel_checks(rel_bias, n_dist, t_every)) return 1;
+  int span = 0;
+  if (n_splits > 1) {
+    DA_REQUIRE(n_splits <= 64, "attn_decode_rel: %d shares (2 to 64 are taken)", n_splits);
+    const long keys = (long)max_blocks * page;
+    span = (int)(((keys + n_splits - 1) / n_splits + DA_WAVE - 1) / DA_WAVE * DA_WAVE);
+    const long need = (long)S * Hq * n_splits * (D + 2) * (long)sizeof(float);
+    DA_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= need,
+               "attn_decode_rel: the workspace holds %ld bytes, %ld are needed", workspace_bytes, need);
+  }
+  if (S == 0) return 0;
+  decode_launch(q, q_ld, cache, block_table, max_blocks, seq_lens, S, Hq, Hkv, D, page, scale, window, out, out_ld,
+                n_splits > 1 ? n_splits : 1, span, (float*)workspace, (hipStream_t)stream, rel_bias, n_dist, t_coef, t_every);
+  DA_CHECK_LAUNCH("attn_decode_rel");
+  return 0;
+}
+#else
 extern "C" int da_attn_decode(const void* q, int q_ld, const void* cache, const int* block_table,
                               int max_blocks, const int* seq_lens, int S, int Hq, int Hkv, int D, int page,
                               float scale, int window, void* out, int out_ld, void* stream) {
@@ -455,3 +524,5 @@ extern "C" int da_attn_decode_split_static(const void* q, int q_ld, const void* 
   DA_CHECK_LAUNCH("attn_decode_split_static");
   return 0;
 }
+
+#endif  // DEC_REL

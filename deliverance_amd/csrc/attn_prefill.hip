@@ -27,9 +27,27 @@
 // a row's sums still depend on its position, the window and KP only; RB x KP is chosen from the
 // step's shape on the host.  Smaller row blocks are for short portions only: every row block of 32
 // reads its keys anew, and on long prompts that traffic, not the longest workgroup, binds.
+//
+// Compiled a second time with PF_REL (attn_prefill_rel.hip) the kernel also takes what some designs put on the
+// scores: a bias by the distance between query and key (a table [Hq][n_dist], 32-bit, the last entry for every
+// larger distance; the head's row sits in LDS, times log2 e) and a query temperature
+// 1 + t_coef * ln(floor((p + 1) / t_every) + 1) that multiplies the row's scale (a lane owns one query row).
+// A tile whose keys all lie n_dist - 1 or more behind the wavefront's first row adds one constant.  The plain
+// build has none of that code.
 #include "common.h"
 #include <da_lane_swap.h>
 #include <type_traits>
+
+#ifdef PF_REL
+#define PF_KERNEL attn_prefill_rel_kernel
+#define PF_REL_MAX_DIST 1024       // entries of the bias row that the workgroup keeps in LDS
+#define PF_REL_PARAMS , const float* __restrict__ rel_bias, int n_dist, float t_coef, int t_every
+#define PF_REL_ARGS , rel_bias, n_dist, t_coef, t_every
+#else
+#define PF_KERNEL attn_prefill_kernel
+#define PF_REL_PARAMS
+#define PF_REL_ARGS
+#endif
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
@@ -46,11 +64,11 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 template <int D16, int RB, int KP, bool BT_LDS>
 // (head sizes up to 64 with four wavefronts: registers held to 256, so that two workgroups share a compute unit)
 __global__ void __launch_bounds__(RB * KP * DA_WAVE, (RB * KP == 4 && D16 <= 4) ? 2 : 1)
-attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
-                    const int* __restrict__ block_table, int max_blocks,
-                    const int* __restrict__ q_start, const int* __restrict__ seq_lens, int seq0,
-                    int Hq, int Hkv, int page, float scale, int window,
-                    bf16_t* __restrict__ out, int out_ld) {
+PF_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
+          const int* __restrict__ block_table, int max_blocks,
+          const int* __restrict__ q_start, const int* __restrict__ seq_lens, int seq0,
+          int Hq, int Hkv, int page, float scale, int window,
+          bf16_t* __restrict__ out, int out_ld PF_REL_PARAMS) {
   constexpr int D = D16 * 16;
   constexpr int DT = (D + 31) / 32;       // 32-dimension tiles of the output
   constexpr int KLD = D + 8;              // padded length of a key row in LDS
@@ -70,6 +88,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   bf16_t (*Ks2)[K_TILE] = (bf16_t (*)[K_TILE])smem;
   bf16_t (*Vs2)[V_TILE] = (bf16_t (*)[V_TILE])(smem + NB * K_TILE * 2);
   __shared__ long long bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];   // a page's place in the cache, in bytes
+#ifdef PF_REL
+  __shared__ float brel[PF_REL_MAX_DIST];       // the head's bias by distance, times log2 e (zeros without a table)
+#endif
 
   // The workgroups with the most keys (the last rows) are launched first, those of every (sequence, head) pair
   // before anybody's second-longest: blockIdx.x, which the dispatcher counts up first, is the pair.  (Counted the
@@ -116,7 +137,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
   float m = -INFINITY, l = 0.f;                 // running maximum (base-2 domain); sum of the weights of this lane half's keys
+#ifdef PF_REL
+  // this lane's row has a scale of its own; the bias row is parked before the first barrier below
+  const float scale2 = scale * 1.4426950408889634f *
+                       (t_every > 0 ? 1.0f + t_coef * logf((float)(((q_ok ? pq : 0) + 1) / t_every + 1)) : 1.0f);
+  const int n_rel = rel_bias ? n_dist : 1;
+  for (int i = t; i < n_rel; i += THREADS) brel[i] = rel_bias ? rel_bias[(size_t)h * n_dist + i] * 1.4426950408889634f : 0.f;
+#else
   const float scale2 = scale * 1.4426950408889634f;
+#endif
 
   // The next tile's keys and values are asked for (into registers) before the current tile is
   // multiplied, so their latency hides behind the arithmetic.  Loads are unconditional (a conditional
@@ -267,6 +296,31 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
       // were loaded as zeros.
       const bool whole = WHOLE || (kt + PF_BK - 1 <= w_first && (window <= 0 || kt >= w_last - window + 1));
       float tmax = -INFINITY;
+#ifdef PF_REL
+      // Scores go to the base-2 domain here, with the row's scale and the bias of each key's distance.
+      const int d0 = (q_ok ? pq : -(1 << 30)) - kt - 4 * hf;      // pq - key for the lane's first key
+      const int e0 = (pq - q_lo) - d0;                             // key - q_lo likewise
+      const bool far = kt + PF_BK - 1 <= w_first - (n_rel - 1);    // every key n_rel - 1 or more behind every row
+      const float bfar = brel[n_rel - 1];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = ks * 32 + 8 * (r / 4) + (r % 4);
+          float b = bfar;
+          if (!far) {
+            const int dist = d0 - c;
+            b = brel[dist < 0 ? 0 : (dist < n_rel ? dist : n_rel - 1)];
+          }
+          float v = __builtin_fmaf(sc[ks][r], scale2, b);
+          if (!whole) {
+            const int lo = min(d0 - c, e0 + c);
+            v += __builtin_bit_cast(float, (lo >> 31) & (int)0xff800000);
+          }
+          sc[ks][r] = v;
+          tmax = fmaxf(tmax, v);
+        }
+#else
       if (whole) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
@@ -287,7 +341,12 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
             tmax = fmaxf(tmax, v);
           }
       }
+#endif
+#ifdef PF_REL
+      tmax = half_max(tmax);                           // over both halves of the wavefront: all 64 keys of the row
+#else
       tmax = half_max(tmax) * scale2;                  // over both halves of the wavefront: all 64 keys of the row
+#endif
       const float m_new = fmaxf(m, tmax);
       const bool any = m_new != -INFINITY;             // a row that has seen no key yet keeps zeros
       const float m_use = any ? m_new : 0.f;           // -inf - 0 stays -inf: weight 0, never NaN
@@ -301,8 +360,13 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
           uint32_t u[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
+#ifdef PF_REL
+            const float p0 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e] - m_use);
+            const float p1 = __builtin_amdgcn_exp2f(sc[ks][kb * 8 + 2 * e + 1] - m_use);
+#else
             const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[ks][kb * 8 + 2 * e], scale2, -m_use));
             const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[ks][kb * 8 + 2 * e + 1], scale2, -m_use));
+#endif
             tsum += p0 + p1;
             u[e] = pack2_bf16(p0, p1);
           }
@@ -443,10 +507,24 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __rest
   }
 }
 
+#ifdef PF_REL
+extern "C" int da_attn_prefill_rel_max_dist() { return PF_REL_MAX_DIST; }
+
+extern "C" int da_attn_prefill_rel(const void* q, int q_ld, const void* cache, const int* block_table,
+                                   int max_blocks, const int* q_start, const int* seq_lens, int seq0, int n_seqs,
+                                   int max_query_len, int Hq, int Hkv, int D, int page, float scale, int window,
+                                   const float* rel_bias, int n_dist, float t_coef, int t_every,
+                                   void* out, int out_ld, int form, void* stream) {
+  DA_REQUIRE(!rel_bias || (n_dist > 0 && n_dist <= PF_REL_MAX_DIST), "attn_prefill_rel: a bias table of %d entries (1 to %d are taken)",
+             n_dist, PF_REL_MAX_DIST);
+  DA_REQUIRE(t_every >= 0, "attn_prefill_rel: bad temperature period %d", t_every);
+  DA_REQUIRE(D <= 128, "attn_prefill_rel: head size %d (up to 128 is taken)", D);
+#else
 extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const int* block_table,
                                int max_blocks, const int* q_start, const int* seq_lens, int seq0, int n_seqs,
                                int max_query_len, int Hq, int Hkv, int D, int page, float scale, int window,
                                void* out, int out_ld, int form, void* stream) {
+#endif
   DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && page > 0 && max_query_len >= 0, "attn_prefill: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_prefill: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attn_prefill: head size %d is not a multiple of 16 up to 256", D);
@@ -487,9 +565,9 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
   // every key a workgroup can see lies within max_blocks pages
   const bool bt_lds = max_blocks <= (chosen == 41 ? PF_BT_MAX : PF_BT_MAX_PHASED);
 #define LAUNCH2(N, RB, KP, L)                                                                                  \
-  hipLaunchKernelGGL((attn_prefill_kernel<N, RB, KP, L>), dim3(Hq * n_seqs, da_ceil_div(max_query_len, 32 * RB)), \
+  hipLaunchKernelGGL((PF_KERNEL<N, RB, KP, L>), dim3(Hq * n_seqs, da_ceil_div(max_query_len, 32 * RB)), \
                      dim3(RB * KP * DA_WAVE), 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, \
-                     max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld)
+                     max_blocks, q_start, seq_lens, seq0, Hq, Hkv, page, scale, window, (bf16_t*)out, out_ld PF_REL_ARGS)
 #define LAUNCH3(N, RB, KP)                \
   do {                                    \
     if (bt_lds) LAUNCH2(N, RB, KP, true); \
@@ -513,7 +591,9 @@ extern "C" int da_attn_prefill(const void* q, int q_ld, const void* cache, const
     break;
   switch (D / 16) {
     LAUNCH_SMALL(1) LAUNCH_SMALL(2) LAUNCH_SMALL(3) LAUNCH_SMALL(4) LAUNCH_MID(5) LAUNCH_MID(6) LAUNCH_MID(7) LAUNCH_MID(8)
+#ifndef PF_REL
     LAUNCH(9) LAUNCH(10) LAUNCH(11) LAUNCH(12) LAUNCH(13) LAUNCH(14) LAUNCH(15) LAUNCH(16)
+#endif
   }
 #undef LAUNCH
 #undef LAUNCH_MID

@@ -30,7 +30,8 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
 # Per source: kernels that read their matrix-core results back at once (softmax between two
 # products) keep them in ordinary vector registers; the default puts them into accumulation
 # registers and moves every value out and in again.
-EXTRA_FLAGS = {"attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+EXTRA_FLAGS = {"attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+               "attn_prefill_rel.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _lib = None
 

@@ -90,6 +90,8 @@ _ARGTYPES = {
     "da_can_fuse_ln": [_I, _I, _I],
     "da_run_step": [_VP, _VP],
     "da_top_logprobs": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP],
+    "da_attn_decode_rel": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
+    "da_attn_prefill_rel": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _I, _VP],
     "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _VP],
@@ -855,16 +857,108 @@ def paged_attention(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, 
         return attention_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, scale, window, out)
 
 
+PREFILL_REL_MAX_DIST = 1024     # entries of a bias row that the prefill kernel keeps in LDS (csrc/attn_prefill.hip)
+PREFILL_REL_MAX_HEAD_DIM = 128
+
+
+def _rel_bias_args(dist_bias, n_heads, name):
+    if dist_bias is None:
+        return None, 0
+    _need(dist_bias.dtype == torch.float32 and dist_bias.is_contiguous() and dist_bias.dim() == 2
+          and dist_bias.shape[0] == n_heads, f"{name}: the bias by distance must be float32 [Hq, n_dist]")
+    return _ptr(dist_bias), dist_bias.shape[1]
+
+
+def attention_decode_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                         n_seqs: int, n_heads: int, scale: float, window: Optional[int],
+                         dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int, out: torch.Tensor,
+                         n_splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``attention_decode`` with a bias by distance and a query temperature on the scores."""
+    Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_decode_rel")
+    _need(q.shape[0] >= n_seqs and out.shape[0] >= n_seqs and block_table.shape[0] >= n_seqs,
+          "attention_decode_rel: fewer rows than sequences")
+    _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= n_seqs, "attention_decode_rel: seq_lens must be int32 [S]")
+    bias_ptr, n_dist = _rel_bias_args(dist_bias, n_heads, "attention_decode_rel")
+    _dev(dist_bias, workspace)
+    ws_bytes = 0
+    if n_splits > 1:
+        need = decode_workspace_floats(n_seqs, n_heads, D, n_splits)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.is_contiguous()
+              and workspace.numel() >= need, f"attention_decode_rel: the workspace must hold {need} float32")
+        ws_bytes = workspace.numel() * 4
+    _check(_lib().da_attn_decode_rel(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table), block_table.shape[1],
+                                     _ptr(seq_lens), n_seqs, n_heads, Hkv, D, page, float(scale), int(window or 0),
+                                     bias_ptr, n_dist, float(temp_coef), int(temp_every), _ptr(out), out.stride(0),
+                                     int(n_splits), _ptr(workspace) if n_splits > 1 else None, ws_bytes, _stream()))
+    return out
+
+
+def attention_prefill_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
+                          seq_lens: torch.Tensor, seq0: int, n_seqs: int, max_query_len: int, n_heads: int, scale: float,
+                          window: Optional[int], dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
+                          out: torch.Tensor, form: int = 0) -> torch.Tensor:
+    """``attention_prefill`` with a bias by distance (up to ``PREFILL_REL_MAX_DIST`` entries a head) and a query
+    temperature on the scores; head sizes up to ``PREFILL_REL_MAX_HEAD_DIM``."""
+    Hkv, page, D = _attn_common(q, cache_slot, block_table, n_heads, out, "attention_prefill_rel")
+    _need(q_start.dtype == torch.int32 and q_start.numel() >= seq0 + n_seqs + 1, "attention_prefill_rel: q_start must be int32 [S+1]")
+    _need(seq_lens.dtype == torch.int32 and seq_lens.numel() >= seq0 + n_seqs, "attention_prefill_rel: seq_lens must be int32 [S]")
+    _need(block_table.shape[0] >= seq0 + n_seqs, "attention_prefill_rel: block table has fewer rows than sequences")
+    _need(q.shape[0] == out.shape[0], "attention_prefill_rel: q and out differ in rows")
+    bias_ptr, n_dist = _rel_bias_args(dist_bias, n_heads, "attention_prefill_rel")
+    _dev(dist_bias)
+    _check(_lib().da_attn_prefill_rel(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table), block_table.shape[1],
+                                      _ptr(q_start), _ptr(seq_lens), seq0, n_seqs, max_query_len, n_heads, Hkv, D, page,
+                                      float(scale), int(window or 0), bias_ptr, n_dist, float(temp_coef), int(temp_every),
+                                      _ptr(out), out.stride(0), form, _stream()))
+    return out
+
+
 def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, n_kv_heads: int,
                         head_dim: int, v_head_dim: int, scale: float, window: Optional[int],
                         dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
                         out: torch.Tensor) -> torch.Tensor:
     """Attention of every row of the step with a bias by distance, a query temperature and values of their own
-    size (each optional).  32-bit, the reference mode and shapes the matrix-core kernels do not take use the
-    plain kernel for all rows."""
+    size (each optional).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
+    bias row that fits the prefill kernel's LDS copy, the one-token sequences go to the decode kernel and the
+    portions to the prefill kernel (their forms with these extras); 32-bit, the reference mode and every other
+    shape use the plain kernel for all rows."""
     bt = ctx.block_tables[group]
-    page = ctx.cache.page_size
-    with _timed("attention_plain", 0, 0, "fp32" if q.dtype == torch.float32 else "bf16"):
+    page = cache_slot.shape[3] if cache_slot.dim() == 5 else ctx.cache.page_size
+    D, nd = head_dim, ctx.n_decode
+    el = cache_slot.element_size()
+    lens, starts = ctx.seq_lens_host, ctx.q_start_host        # for the profiler's cost model only
+
+    def cost(first, last):
+        if not KernelProfiler.enabled or not lens:
+            return 0, 0
+        keys = pairs = rows = 0
+        for s_ in range(first, last):
+            t = starts[s_ + 1] - starts[s_]
+            n = lens[s_]
+            keys += n
+            rows += t
+            pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
+        return (keys * n_kv_heads * (D + v_head_dim) * el + rows * n_heads * (D + v_head_dim) * el,
+                2 * pairs * n_heads * (D + v_head_dim))
+
+    tuned = (_MODE == "tuned" and q.dtype == torch.bfloat16 and v_head_dim == D and D % 16 == 0
+             and D <= PREFILL_REL_MAX_HEAD_DIM and cache_slot.dim() == 5 and q.stride(0) % 8 == 0
+             and q.data_ptr() % 16 == 0 and (dist_bias is None or dist_bias.shape[1] <= PREFILL_REL_MAX_DIST))
+    if tuned:
+        if nd:
+            n_splits = decode_splits(nd, n_heads, bt.shape[1], page)
+            ws = None
+            if n_splits > 1:
+                ws = ctx.buf("decode_partial", 1, decode_workspace_floats(nd, n_heads, D, n_splits), torch.float32)
+            with _timed("attention_decode", *cost(0, nd)):
+                attention_decode_rel(q, cache_slot, bt, ctx.seq_lens, nd, n_heads, scale, window, dist_bias, temp_coef,
+                                     temp_every, out, n_splits, ws)
+        if ctx.n_seqs > nd:
+            with _timed("attention_prefill", *cost(nd, ctx.n_seqs)):
+                attention_prefill_rel(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
+                                      ctx.max_query_len, n_heads, scale, window, dist_bias, temp_coef, temp_every, out)
+        return out
+    with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_rel_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, n_kv_heads, head_dim,
                                  v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out)
 

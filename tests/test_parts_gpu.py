@@ -72,7 +72,7 @@ def test_norm_part(dtype):
     want = P.layer_norm(x.double().cpu().numpy(), w.double().numpy(), None, 1e-6)
     assert np.abs(got.double().cpu().numpy() - want).max() < TOL[dtype]
     with pytest.raises(KeyError, match="no norm of kind"):
-        build_norm(NormSpec("rmsnorm", E, 1e-6), {"weight": w}, dtype, DEV)
+        build_norm(NormSpec("groupnorm", E, 1e-6), {"weight": w}, dtype, DEV)
 
 
 def test_learned_positions_part():
