@@ -26,6 +26,10 @@ struct LnPrologue {
   const void* b;
   int b_dtype;
   float eps;
+  // LayerNorm: center 1, gain_offset 0.  A root-mean-square norm is the same arithmetic with the mean taken
+  // as zero (center 0), no bias, and a gain of gain_offset + g (1 + g for gains stored around zero).
+  float center;
+  float gain_offset;
 };
 
 __device__ __forceinline__ void load8_param(const void* p, int dtype, int i, float* o) {
@@ -96,7 +100,7 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
       v[i] = *(const float4*)(xr + (c < K ? c : 0));          // never a conditional load, nor a value replaced
       s += (c < K ? 1.f : 0.f) * ((v[i].x + v[i].y) + (v[i].z + v[i].w));
     }
-    const float mean = wave_sum(s) / (float)K;
+    const float mean = wave_sum(s) / (float)K * ln.center;
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < FZ_VPL; ++i) {
@@ -149,8 +153,8 @@ gemm_ln_skinny_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epil
         uint32_t pk[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float y0 = (xs[2 * e] - mean[i]) * rstd[i] * gg[u][2 * e];
-          float y1 = (xs[2 * e + 1] - mean[i]) * rstd[i] * gg[u][2 * e + 1];
+          float y0 = (xs[2 * e] - mean[i]) * rstd[i] * (gg[u][2 * e] + ln.gain_offset);
+          float y1 = (xs[2 * e + 1] - mean[i]) * rstd[i] * (gg[u][2 * e + 1] + ln.gain_offset);
           if (ln.b) { y0 += bb[u][2 * e]; y1 += bb[u][2 * e + 1]; }
           pk[e] = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
         }
@@ -282,7 +286,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
       const int c = (lane + i * 64) * 4;
       sum += (c < K ? 1.f : 0.f) * ((sv[j][i].x + sv[j][i].y) + (sv[j][i].z + sv[j][i].w));
     }
-    const float mean = wave_sum(sum) / (float)K;
+    const float mean = wave_sum(sum) / (float)K * ln.center;
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < RV; ++i) {
@@ -308,7 +312,7 @@ gemm_ln_rows_kernel(LnPrologue ln, const bf16_t* __restrict__ w, int ldw, Epilog
       float y[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        y[e] = (xs[e] - mean) * rstd * g4[e];
+        y[e] = (xs[e] - mean) * rstd * (g4[e] + ln.gain_offset);
         if (ln.b) y[e] += b4[e];
       }
       uint2 pk = make_uint2((uint32_t)f32_to_bf16(y[0]) | ((uint32_t)f32_to_bf16(y[1]) << 16),
@@ -384,11 +388,11 @@ static void launch_fused(int mt, dim3 grid, hipStream_t s, const LnPrologue& ln,
   else hipLaunchKernelGGL((gemm_ln_skinny_kernel<2, NW, UN>), grid, dim3(NW * 64), 0, s, ln, W, ldw, ep, kv, M, N, K);
 }
 
-extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, int g_dtype, const void* b,
-                               int b_dtype, float eps, const void* w, int ldw, const void* bias, int bias_dtype,
-                               int act, void* out, int out_dtype, int ldo, int M, int N, int K, void* kv_cache,
-                               const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
-                               void* stream) {
+static int gemm_bf16_norm(const float* x, const int* rows, const void* g, int g_dtype, const void* b,
+                          int b_dtype, float eps, float center, float gain_offset, const void* w, int ldw,
+                          const void* bias, int bias_dtype, int act, void* out, int out_dtype, int ldo, int M, int N,
+                          int K, void* kv_cache, const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
+                          void* stream) {
   DA_REQUIRE(M > 0 && M <= 32 && N > 0 && K > 0, "gemm_bf16_ln: takes 1..32 rows (M=%d N=%d K=%d)", M, N, K);
   DA_REQUIRE(K % 8 == 0 && K <= 256 * FZ_VPL && ldw % 8 == 0 && ldw >= K && ldo >= N,
              "gemm_bf16_ln: K must be a multiple of 8 up to %d (K=%d ldw=%d)", 256 * FZ_VPL, K, ldw);
@@ -400,7 +404,7 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
     DA_REQUIRE(out_dtype == DA_BF16 && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N && page > 0,
                "gemm_bf16_ln: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);
   }
-  LnPrologue ln{x, rows, g, g_dtype, b, b_dtype, eps};
+  LnPrologue ln{x, rows, g, g_dtype, b, b_dtype, eps, center, gain_offset};
   Epilogue ep{bias, bias_dtype, act, 0, out, out_dtype, ldo};
   KvScatter kv{kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page};
   dim3 grid(da_ceil_div(N, FZ_COLS));
@@ -445,4 +449,23 @@ extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, i
     launch_fused<8, 2>(mt, grid, s, ln, (const bf16_t*)w, ldw, ep, kv, M, N, K);
   DA_CHECK_LAUNCH("gemm_bf16_ln");
   return 0;
+}
+
+extern "C" int da_gemm_bf16_ln(const float* x, const int* rows, const void* g, int g_dtype, const void* b,
+                               int b_dtype, float eps, const void* w, int ldw, const void* bias, int bias_dtype,
+                               int act, void* out, int out_dtype, int ldo, int M, int N, int K, void* kv_cache,
+                               const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page,
+                               void* stream) {
+  return gemm_bf16_norm(x, rows, g, g_dtype, b, b_dtype, eps, 1.0f, 0.0f, w, ldw, bias, bias_dtype, act, out, out_dtype,
+                        ldo, M, N, K, kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page, stream);
+}
+
+// The same kernels with a root-mean-square norm in front of the product:
+//   out = act((x / sqrt(mean(x^2) + eps) * (gain_offset + g)) @ w.T + bias)
+extern "C" int da_gemm_bf16_rms(const float* x, const int* rows, const void* g, int g_dtype, float gain_offset,
+                                float eps, const void* w, int ldw, const void* bias, int bias_dtype, int act,
+                                void* out, int out_dtype, int ldo, int M, int N, int K, void* kv_cache,
+                                const int* slot_map, int q_cols, int kv_cols, int Hkv, int D, int page, void* stream) {
+  return gemm_bf16_norm(x, rows, g, g_dtype, nullptr, 0, eps, 0.0f, gain_offset, w, ldw, bias, bias_dtype, act, out,
+                        out_dtype, ldo, M, N, K, kv_cache, slot_map, q_cols, kv_cols, Hkv, D, page, stream);
 }

@@ -12,7 +12,7 @@
 // used is decided on the device, so a step can be recorded.  A pair's result does not depend on its slot:
 // sums over k run in the same order for every row.  Expert weights are stacked: gate | up as
 // [n_experts][2 F][K] (gate rows first), down as [n_experts][width][F].
-#include "common.h"
+#include "gemm_common.h"
 
 #define MOE_MAX_EXPERTS 1024
 
@@ -168,7 +168,6 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
       if (n >= F) continue;
       const size_t o = (size_t)(m0 + r) * ldo + n;
       if (GATED) {
-        // the gate is rounded as a product of its own would be before the activation sees it
         if (DTypeOf<T>::value == DA_BF16)
           from_f32(&((T*)out)[o], apply_act_bf16(acc[0][i][j], act) * acc[1][i][j]);
         else
@@ -234,5 +233,116 @@ extern "C" int da_moe_combine(const float* out, int ldo, const int* slot_of_pair
   hipLaunchKernelGGL(moe_combine_kernel, dim3(da_ceil_div((long)N * width, 256)), dim3(256), 0, (hipStream_t)stream, out,
                      ldo, slot_of_pair, weights, uniform, top, y, ldy, N, width, accumulate);
   DA_CHECK_LAUNCH("moe_combine");
+  return 0;
+}
+
+// ---- the grouped products on the matrix cores (bfloat16) ---------------------------------------------------
+// A workgroup of four wavefronts owns a tile of 32 slots x 64 columns of one expert: wavefront v the columns
+// 16 v .. 16 v + 15 of both blocks of 16 rows, with MFMA 16x16x32.  Operands go from memory into the lanes'
+// fragments (a lane's 16 bytes are 8 consecutive k of one row), four k-steps of 32 asked for at once; with
+// few rows an expert, as in decoding, the kernel streams the expert's weights once.  GATED: the gate and up
+// rows of the same columns are multiplied side by side and out = act(g) * u leaves in bfloat16; else one
+// product leaves in 32-bit.  A row's sums run over k in ascending order whatever else is in the step.
+#define MM_ROWS 32
+#define MM_COLS 64
+#define MM_UNROLL 4
+
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
+                const int* __restrict__ tile_expert, const bf16_t* __restrict__ w, void* __restrict__ out, int ldo,
+                int K, int F, int act) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
+  const int fr = lane % 16, fk = (lane / 16) * 8;
+  const int m0 = blockIdx.y * MM_ROWS, n0 = blockIdx.x * MM_COLS + wave * 16;
+  if (n0 >= F) return;
+  // the rows of a: gathered by slot for the first product (a padding slot reads row 0 and is never stored),
+  // the slot's own row for the second
+  const bf16_t* ap[2];
+  int srow[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    srow[i] = row_of_slot[m0 + i * 16 + fr];
+    const int r = GATED ? (srow[i] >= 0 ? srow[i] : 0) : m0 + i * 16 + fr;
+    ap[i] = a + (size_t)r * lda + fk;
+  }
+  const int wcol = n0 + fr < F ? n0 + fr : 0;
+  const bf16_t* wg = w + ((size_t)e * (GATED ? 2 : 1) * F + wcol) * K + fk;
+  const bf16_t* wu = wg + (size_t)F * K;
+  floatx4 acc[2][GATED ? 2 : 1];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int g = 0; g < (GATED ? 2 : 1); ++g) acc[i][g] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int k0 = 0; k0 < K; k0 += 32 * MM_UNROLL) {
+    uint4 av[MM_UNROLL][2], wv[MM_UNROLL][GATED ? 2 : 1];
+#pragma unroll
+    for (int u = 0; u < MM_UNROLL; ++u) {
+      const int k = k0 + u * 32;
+      const int ks = (k + fk < K) ? k : -fk;            // past K: the row's first chunk, met by zeros in a
+      av[u][0] = load16(ap[0] + ks);
+      av[u][1] = load16(ap[1] + ks);
+      wv[u][0] = load16(wg + ks);
+      if (GATED) wv[u][GATED ? 1 : 0] = load16(wu + ks);
+    }
+#pragma unroll
+    for (int u = 0; u < MM_UNROLL; ++u) {
+      const bool kin = k0 + u * 32 + fk < K;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint4 x = kin ? av[u][i] : zero;
+#pragma unroll
+        for (int g = 0; g < (GATED ? 2 : 1); ++g)
+          acc[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x),
+                                                              __builtin_bit_cast(bf16x8_t, wv[u][g]), acc[i][g], 0, 0, 0);
+      }
+    }
+  }
+  // acc[i][.][r] is row 16 i + 4 (lane / 16) + r of the tile, column n0 + fr
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * (lane / 16) + r;
+      const int used = row_of_slot[m0 + i * 16 + row];
+      if (used < 0 || n0 + fr >= F) continue;
+      const size_t o = (size_t)(m0 + i * 16 + row) * ldo + n0 + fr;
+      if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(acc[i][0][r], act) * acc[i][GATED ? 1 : 0][r]);
+      else ((float*)out)[o] = acc[i][0][r];
+    }
+}
+
+static int moe_mfma_checks(const void* a, int lda, const void* w, int K, const char* name) {
+  DA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0,
+             "%s: K and the row length of a must be multiples of 8, operands 16-byte aligned", name);
+  return 0;
+}
+
+extern "C" int da_moe_tile_rows_mfma() { return MM_ROWS; }
+
+extern "C" int da_moe_gated_mfma(const void* a, int lda, const int* row_of_slot, const int* tile_expert, const void* w,
+                                 void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
+  DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_mfma: bad sizes");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "moe_gated_mfma: unknown activation %d", act);
+  if (moe_mfma_checks(a, lda, w, K, "moe_gated_mfma")) return 1;
+  if (T_cap == 0) return 0;
+  hipLaunchKernelGGL((moe_mfma_kernel<true>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act);
+  DA_CHECK_LAUNCH("moe_gated_mfma");
+  return 0;
+}
+
+extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot, const int* tile_expert, const void* w,
+                                float* out, int ldo, int T_cap, int F, int width, void* stream) {
+  DA_REQUIRE(T_cap >= 0 && F > 0 && width > 0 && ldm >= F && ldo >= width, "moe_down_mfma: bad sizes");
+  if (moe_mfma_checks(mid, ldm, w, F, "moe_down_mfma")) return 1;
+  if (T_cap == 0) return 0;
+  hipLaunchKernelGGL((moe_mfma_kernel<false>), dim3(da_ceil_div(width, MM_COLS), T_cap), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F,
+                     width, 0);
+  DA_CHECK_LAUNCH("moe_down_mfma");
   return 0;
 }

@@ -80,6 +80,8 @@ _ARGTYPES = {
     "da_gemm_wide_choice": [_I, _I, _I],
     "da_gemm_bf16_ln": [_VP, _VP, _VP, _I, _VP, _I, _F, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP,
                         _I, _I, _I, _I, _I, _VP],
+    "da_gemm_bf16_rms": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _I, _VP, _VP,
+                         _I, _I, _I, _I, _I, _VP],
     "da_kv_write": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_attn_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
     "da_attn_decode": [_VP, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
@@ -101,6 +103,8 @@ _ARGTYPES = {
     "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP],
     "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
+    "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_down_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_combine": [_VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _I, _I, _VP],
 }
 _LIB = None
@@ -329,6 +333,7 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------- experts
 MOE_TILE_ROWS = 64       # rows of a tile of the plain grouped products
+MOE_TILE_ROWS_MFMA = 32  # ... of the matrix-core grouped products (csrc/moe.hip)
 
 
 def moe_slot_space(n_tokens: int, top: int, n_experts: int, tile: int):
@@ -712,6 +717,37 @@ def linear_ln(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_w
     return out
 
 
+def linear_rms(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, norm_weight: torch.Tensor,
+               gain_offset: float, eps: float, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+               act: Optional[str] = None, kv_cache: Optional[torch.Tensor] = None,
+               slot_map: Optional[torch.Tensor] = None, q_cols: int = 0) -> torch.Tensor:
+    """``linear_ln`` with a root-mean-square norm in front of the product:
+    out = act((x[rows] / sqrt(mean(x^2) + eps) * (gain_offset + norm_weight)) @ w.T + bias), for steps that
+    ``can_fuse_ln`` takes."""
+    _dev(x, rows, norm_weight, w, bias, out, kv_cache, slot_map)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "linear_rms: x must be contiguous float32")
+    _rows_2d(w, "w"); _rows_2d(out, "out")
+    N, K = w.shape
+    _need(x.shape[1] == K and norm_weight.numel() == K, "linear_rms: widths differ")
+    _need(w.dtype == torch.bfloat16, "linear_rms: w must be bfloat16")
+    _need(0 < n_rows <= FUSED_LN_KERNEL_MAX_ROWS and out.shape[0] >= n_rows and out.shape[1] == N, "linear_rms: bad row count")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "linear_rms: fewer rows in x than asked")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "linear_rms: rows must be int32")
+    _need(bias is None or bias.numel() == N, "linear_rms: bias length differs from N")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"linear_rms: unknown activation {act!r}")
+    kvp = _kv_args(kv_cache, slot_map, q_cols, n_rows, N, out, "linear_rms")
+    with _timed("norm_product_fused", n_rows * K * 4 + _nbytes(w, bias, norm_weight) + n_rows * N * out.element_size(),
+                2 * n_rows * N * K):
+        _check(_lib().da_gemm_bf16_rms(
+            _ptr(x), _ptr(rows), _ptr(norm_weight), _dt(norm_weight), float(gain_offset), float(eps), _ptr(w), w.stride(0),
+            _ptr(bias), _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(out), _dt(out), out.stride(0),
+            n_rows, N, K, *kvp, _stream()))
+    return out
+
+
 def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -971,18 +1007,40 @@ def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor,
     return gated_act(gu, mid, act)
 
 
+def _moe_mfma_ok(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> bool:
+    return (_MODE == "tuned" and h.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and h.shape[1] % 8 == 0
+            and h.stride(0) % 8 == 0 and down.shape[2] % 8 == 0 and h.data_ptr() % 16 == 0
+            and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0)
+
+
 def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
                     n_experts: int, top: int, weight: float, act: str, x: torch.Tensor, accumulate: bool) -> torch.Tensor:
-    """x (+)= sum_k weight * expert_{table[token, k]}(h): route, two grouped products, combine."""
+    """x (+)= sum_k weight * expert_{table[token, k]}(h): route, two grouped products, combine.  bfloat16 steps
+    run the grouped products on the matrix cores; 32-bit and the reference mode use the plain ones."""
     N, width = h.shape
     inner = down.shape[2]
-    tile = MOE_TILE_ROWS
+    mfma = _moe_mfma_ok(h, gate_up, down)
+    tile = MOE_TILE_ROWS_MFMA if mfma else MOE_TILE_ROWS
     tiles, rows = moe_slot_space(N, top, n_experts, tile)
     ints = ctx.buf("moe_route", N * top + rows + tiles, 1, torch.int32).view(-1)
     slot_of_pair, row_of_slot, tile_expert = ints[:N * top], ints[N * top:N * top + rows], ints[N * top + rows:]
     moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
     mid = ctx.buf("moe_mid", rows, inner, h.dtype)
     pair_out = ctx.buf("moe_out", rows, width, torch.float32)
-    moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
-    moe_down_ref(mid, row_of_slot, tile_expert, down, pair_out, tiles)
+    if mfma:
+        _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, 2 * inner, width)
+              and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
+        _dev(h, gate_up, down)
+        # every expert's weights once (decode: what the step must move), the pairs' rows in and out
+        nb = N * top * (width * 2 + inner * 2) + min(n_experts, N * top) * 2 * inner * width * 2
+        with _timed("experts_gated", nb, 4 * N * top * inner * width):
+            _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
+                                            _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], _stream()))
+        nb = N * top * (inner * 2 + width * 4) + min(n_experts, N * top) * inner * width * 2
+        with _timed("experts_down", nb, 2 * N * top * inner * width):
+            _check(_lib().da_moe_down_mfma(_ptr(mid), mid.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(down),
+                                           _ptr(pair_out), pair_out.stride(0), tiles, inner, width, _stream()))
+    else:
+        moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
+        moe_down_ref(mid, row_of_slot, tile_expert, down, pair_out, tiles)
     return moe_combine(pair_out, slot_of_pair, None, weight, top, x, accumulate)

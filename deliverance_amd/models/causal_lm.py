@@ -93,9 +93,13 @@ class CausalLM:
         if n_want == 0:
             return logits
         ln = None if self.final_norm is None else self.final_norm.fusable_params()
+        rms = None if self.final_norm is None or ln is not None else getattr(self.final_norm, "rms_params", lambda: None)()
         if ln is not None and ops.can_fuse_ln(n_want, x, self.head_weight):
             gain, bias, eps = ln                   # few wanted rows: norm and head in one kernel
             ops.linear_ln(x, want_rows, n_want, gain, bias, eps, self.head_weight, None, logits)
+        elif rms is not None and ops.can_fuse_ln(n_want, x, self.head_weight):
+            gain, offset, eps = rms
+            ops.linear_rms(x, want_rows, n_want, gain, offset, eps, self.head_weight, None, logits)
         else:
             if self.final_norm is not None:
                 e = self.final_norm.forward(ctx, x, rows=want_rows, n_rows=n_want, out_name="final_norm")

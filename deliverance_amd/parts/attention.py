@@ -99,20 +99,28 @@ class CausalSelfAttention(Mixer):
         keys and values of one size)."""
         return self.position is None and self.v_head_dim == self.head_dim
 
-    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call) -> bool:
-        """Small steps: LayerNorm, the q|k|v projection and the cache write in one kernel."""
+    normed_into = True
+
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call, into=None) -> bool:
+        """Small steps: the norm in front (LayerNorm or a root-mean-square norm), the q|k|v projection and the
+        cache write in one kernel.  The result joins ``into`` (the stream ``x`` itself when None)."""
         N = x.shape[0]
         ln = norm.fusable_params()
-        if ln is None or not self._epilogue_write() or not ops.can_fuse_ln(N, x, self.qkv_weight):
+        rms = getattr(norm, "rms_params", lambda: None)() if ln is None else None
+        if (ln is None and rms is None) or not self._epilogue_write() or not ops.can_fuse_ln(N, x, self.qkv_weight):
             return False
-        gain, bias, eps = ln
         qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
-        ops.linear_ln(x, None, N, gain, bias, eps, self.qkv_weight, self.qkv_bias, qkv,
-                      kv_cache=slot if call.write else None, slot_map=ctx.slot_maps[group] if call.write else None,
-                      q_cols=self.q_cols)
-        self._attend(ctx, qkv, x, slot, group, call)
+        kv = dict(kv_cache=slot if call.write else None, slot_map=ctx.slot_maps[group] if call.write else None,
+                  q_cols=self.q_cols)
+        if ln is not None:
+            gain, bias, eps = ln
+            ops.linear_ln(x, None, N, gain, bias, eps, self.qkv_weight, self.qkv_bias, qkv, **kv)
+        else:
+            gain, offset, eps = rms
+            ops.linear_rms(x, None, N, gain, offset, eps, self.qkv_weight, self.qkv_bias, qkv, **kv)
+        self._attend(ctx, qkv, x if into is None else into, slot, group, call)
         return True
 
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:

@@ -52,12 +52,14 @@ class Block:
                 ops.fill_zero(target)
         ctx.part_accumulate = not stores
         try:
-            # A part may offer `forward_normed(ctx, norm, x, ...)`: it then applies the norm in front
-            # of it itself (fused into its first product) and returns True, or returns False to
-            # decline this step.  That needs the part's input and the tensor it adds into to be the same.
+            # A part may offer `forward_normed(ctx, norm, x, ..., into=None)`: it then applies the norm in
+            # front of it itself (fused into its first product) and returns True, or returns False to
+            # decline this step.  `into` is where its result goes when that is not the stream itself; a
+            # part that declares `normed_into` takes it.
             if h_ready is not None:
                 run(h_ready, target)
-            elif not (not own and pre is not None and run_normed is not None and run_normed(pre)):
+            elif not (pre is not None and run_normed is not None and (not own or getattr(part, "normed_into", False))
+                      and run_normed(pre, target if own else None)):
                 run(Block._normed(ctx, x, pre), target)
         finally:
             ctx.part_accumulate = True
@@ -73,7 +75,8 @@ class Block:
         fused = getattr(self.mixer, "forward_normed", None)
         h_ff = self._part(ctx, x, self.pre_mixer_norm, self.post_mixer_norm,
                           lambda h, into: self.mixer.forward(ctx, h, into, call),
-                          None if fused is None else (lambda norm: fused(ctx, norm, x, call)), part=self.mixer,
+                          None if fused is None else (lambda norm, into: fused(ctx, norm, x, call) if into is None
+                                                      else fused(ctx, norm, x, call, into=into)), part=self.mixer,
                           next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else self.pre_ff_norm)
         if ctx.debug_hook is not None:
             ctx.emit(call.layer, "post_attention_residual", x)
@@ -81,7 +84,8 @@ class Block:
             fused = getattr(self.feed_forward, "forward_normed", None)
             self._part(ctx, x, self.pre_ff_norm, self.post_ff_norm,
                        lambda h, into: self.feed_forward.forward(ctx, h, into),
-                       None if fused is None else (lambda norm: fused(ctx, norm, x)), part=self.feed_forward,
+                       None if fused is None else (lambda norm, into: fused(ctx, norm, x) if into is None
+                                                   else fused(ctx, norm, x, into=into)), part=self.feed_forward,
                        h_ready=h_ff)
             if ctx.debug_hook is not None:
                 ctx.emit(call.layer, "post_ff_residual", x)
