@@ -13,6 +13,11 @@ and 64; `prefill`: one step of 2 x 1,024 tokens) and then, into the same line, G
 sizes (decode at batch 1, 8, 64 and the same prefill) and the mixed workload at GPT-2 355M layer
 sizes (64 requests at once, prompt portions of 512 tokens beside the others' decoding), each with
 its fraction of the roofline; `--no-extra` leaves those two out.  Prints ONE JSON line.
+
+`--design virudra` measures another design beside GPT-2 at equal sizes instead (width, heads, head size, layers,
+vocabulary, feed-forward parameters that a token uses): decode at batch 1, 8 and 64 and the prefill of 2 x 1,024
+tokens for both, at the layer sizes of GPT-2 124M and 355M, one JSON line; with `--profile-stages` also both
+models' kernel tables (stderr).
 """
 import argparse
 import json
@@ -97,6 +102,10 @@ def engine_from_gpu_weights(cfg, dtype, seats, seed=0, **kw):
     for d in arch.declare_tensors(mc):
         if d.optional:
             continue
+        if d.init == "distinct_ints":                  # (a table of integers: drawn as the random-weights mode draws it)
+            from deliverance_amd.weights.loader import draw_tensor
+            tensors[d.name] = draw_tensor(d, seed).to("cuda:0")
+            continue
         t = torch.randn(d.shape, generator=g, device="cuda:0", dtype=torch.float32) * d.std
         if d.init == "ones_plus_normal":
             t += 1.0
@@ -110,6 +119,80 @@ def engine_from_gpu_weights(cfg, dtype, seats, seed=0, **kw):
     pool = kw.pop("max_cached_tokens", max(seats, 2) * cfg["n_positions"])
     ec = EngineConfig(dtype=dtype, max_num_seqs=max(seats, 2), max_cached_tokens=pool, **kw)
     return CausalLanguageModel(model, ec)
+
+
+def virudra_config(name, n_positions=1024):
+    """A Virudra of GPT-2 ``name``'s sizes: as many layers, heads and key heads of the same head size, dense gated
+    feed-forwards and mixtures of 8 experts (2 a token) in turn whose matrices that a token uses hold what GPT-2's
+    two hold (3 x width x 8/3 width), a bias table of 32 rows up to a distance of 512, no loop."""
+    g = MODELS[name]
+    E, H = g["n_embd"], g["n_head"]
+    D = E // H
+    F = (8 * E // 3 + 63) // 64 * 64
+    mixer = {"heads": H, "kv_heads": H, "dim": D, "vdim": D, "scale": D ** -0.5, "bias_max": 512, "bias_buckets": 32,
+             "q_temp": {"coef": 0.1, "every": 256}}
+    layers = [{"type": "attention", "mixer": mixer,
+               "mlp": {"kind": "dense", "ff": F} if i % 2 == 0 else
+                      {"kind": "moe", "expert": {"ff": F // 2}, "router": {"experts": 8, "top": 2}}}
+              for i in range(g["n_layer"])]
+    return {"architecture": "Virudra", "vocab": 50257, "width": E, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": layers, "max_positions": n_positions,
+            # what decode_run and prefill_run read
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": g["n_layer"], "n_embd": E, "ff": F}
+
+
+def virudra_weight_bytes(c, el, batch):
+    """What a decode step must read of the weights: every matrix once, of the experts as many as ``batch`` tokens
+    can choose (2 each of 8)."""
+    E, F, V = c["width"], c["ff"], c["vocab"]
+    n = 0
+    for L in c["layers"]:
+        n += 4 * E * E
+        n += 3 * E * F if L["mlp"]["kind"] == "dense" else min(8, 2 * batch) * 3 * E * (F // 2)
+    return (n + V * E) * el
+
+
+def virudra_step_flops(c, seq_lens_new):
+    E, F, V = c["width"], c["ff"], c["vocab"]
+    n = sum(seq_lens_new)
+    gemm = 2 * n * (4 * E * E + 3 * E * F) * len(c["layers"]) + 2 * len(seq_lens_new) * E * V
+    attn = sum(4 * sum(i + 1 for i in range(t)) * E * len(c["layers"]) for t in seq_lens_new)
+    return gemm + attn
+
+
+def design_compare(args):
+    """Decode and prefill of Virudra beside GPT-2 at equal sizes; one JSON line."""
+    import numpy as np
+    el, dkey = 2, "bf16"
+    out = {"metric": "decode tok/s at batch 8 of Virudra at GPT-2 124M layer sizes (beside GPT-2 itself: see points)",
+           "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": dkey, "steps": args.steps, "warmup": args.warmup,
+           "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", "points": {}, "points_frac": {}}
+    for size in ("124m", "355m"):
+        for design in ("gpt2", "virudra"):
+            rng = np.random.default_rng(0)
+            cfg = model_config(size) if design == "gpt2" else virudra_config(size)
+            model = engine_from_gpu_weights(cfg, "bfloat16", 64, kernels=args.kernels)
+            key = f"{design}_{size}"
+            for b in (1, 8, 64):
+                steps = min(args.steps, 128)
+                d, cm = decode_run(model, cfg, rng, b, args.prompt_len, steps, 8)
+                out["points"][f"{key}_decode_b{b}"] = round(b * steps / d, 1)
+                wb = weight_bytes(cfg, el) if design == "gpt2" else virudra_weight_bytes(cfg, el, b)
+                kv = 2 * cfg["n_embd"] * el * cfg["n_layer"]
+                out["points_frac"][f"{key}_decode_b{b}"] = round((wb + b * cm * kv) / (d / steps) / 1e9 / HBM_GBS, 4)
+            pf = prefill_run(model, cfg, rng, dkey, flops=None if design == "gpt2" else virudra_step_flops(cfg, [1024, 1024]))
+            out["points"][f"{key}_prefill_2048"] = pf["value"]
+            out["points_frac"][f"{key}_prefill_2048"] = pf["frac"]
+            if args.profile_stages:
+                print(f"==== {key}", file=sys.stderr)
+                kernel_table(model, cfg, rng, args.batch, args.prompt_len)
+            del model
+    out["value"] = out["points"]["virudra_124m_decode_b8"]
+    out["config"] = {"model": "virudra at gpt2-124m and gpt2-355m layer sizes", "global_batch": 8, "prompt_len": args.prompt_len,
+                     "virudra": "heads = key heads, head size 64, gated feed-forward of 8/3 width and 8 experts (2 a token) of "
+                                "half that in turn, bias rows 32 up to distance 512, temperature every 256", "parallelism": "single-gpu"}
+    print(json.dumps(out))
+    return 0
 
 
 def decode_run(model, cfg, rng, batch, prompt_len, steps, warmup):
@@ -146,7 +229,7 @@ def decode_run(model, cfg, rng, batch, prompt_len, steps, warmup):
     return dt, ctx_mean
 
 
-def prefill_run(model, cfg, rng, dkey, n_prompts=2, length=1024):
+def prefill_run(model, cfg, rng, dkey, n_prompts=2, length=1024, flops=None):
     """``n_prompts`` x ``length``-token prompts (2 x 1,024 unless asked otherwise) in ONE step of the engine's step
     function, logits at the last row of each."""
     import torch
@@ -163,7 +246,7 @@ def prefill_run(model, cfg, rng, dkey, n_prompts=2, length=1024):
         for e in entries:
             model.cache.manager.close(e.rid)
     t = min(times[2:])
-    fl = step_flops(cfg, [length] * n_prompts)
+    fl = flops if flops is not None else step_flops(cfg, [length] * n_prompts)
     n = n_prompts * length
     return {"value": round(n / t, 1), "tokens": n, "ms": round(t * 1e3, 3), "frac": round(fl / t / PEAK_FLOPS[dkey], 4)}
 
@@ -239,6 +322,9 @@ def main():
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
                          "requests out of the cache and back, which the line reports as preemptions)")
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra"],
+                    help="virudra: that design beside GPT-2 at equal sizes (decode at batch 1, 8, 64 and the prefill of 2,048 "
+                         "tokens, at 124M and 355M layer sizes) instead of the default workload")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="mixed: only the mixed workload, on --model (64 requests with prompts of 16 to 895 tokens arrive at "
                          "once, prompt portions of 512 tokens run beside the decoding of the others, 128 new tokens each)")
@@ -250,6 +336,8 @@ def main():
     import numpy as np
     from deliverance_amd.random_model import random_model
 
+    if args.design == "virudra":
+        return design_compare(args)
     cfg = model_config(args.model, args.layers, args.n_positions)
     full_layers = MODELS[args.model]["n_layer"]
     el = 2 if args.dtype == "bfloat16" else 4
