@@ -193,11 +193,20 @@ tile_epilogue(floatx16 (&acc)[BM / WM / 32][BN / WN / 32], const float (&bias)[B
   }
 }
 
+// Grouped products: the rows of a come in groups of `rows` (a multiple of the tile's rows), and group i is
+// multiplied with the matrix w + tile_group[i] * stride (a stack of matrices of one shape: the experts of a
+// feed-forward); a group whose entry is negative is not used and its tiles leave at once.  No grouping: null.
+struct Grouping {
+  const int* tile_group;
+  long stride;
+  int rows;
+};
+
 template <int BM, int BN, int WM, int WN, int PF_SLABS, int ACT, int OUTMODE, bool KTAIL>
 __device__ __forceinline__ void
 gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
                const Epilogue& ep, const KvScatter& kv, int M, int N, int K, int tiles_m, int tiles_n,
-               char* smem) {
+               char* smem, const Grouping& gr) {
   bf16_t (*As)[BM * LDS_LD] = (bf16_t (*)[BM * LDS_LD])smem;
   bf16_t (*Ws)[BN * LDS_LD] = (bf16_t (*)[BN * LDS_LD])(smem + 2 * BM * LDS_LD * sizeof(bf16_t));
   constexpr int THREADS = WM * WN * 64;
@@ -218,6 +227,11 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
   }
   const int tm = pid % tiles_m, tn = pid / tiles_m;
   const int m0 = tm * BM, n0 = tn * BN;
+  if (gr.tile_group) {                      // (the same for the whole workgroup, before any barrier)
+    const int g = gr.tile_group[m0 / gr.rows];
+    if (g < 0) return;
+    w += (size_t)g * gr.stride;
+  }
 
   const int t = threadIdx.x, lane = t % 64, wave = t / 64;
   const int wm = (wave % WM) * (BM / WM), wn = (wave / WM) * (BN / WN);
@@ -350,37 +364,37 @@ gemm_tile_body(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__
 template <int BM, int BN, int WM, int WN, int PF, int ACT, int OUTMODE>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w, int ldw,
-                 Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n) {
+                 Epilogue ep, KvScatter kv, int M, int N, int K, int tiles_m, int tiles_n, Grouping gr) {
   // two buffers of a slab of a and of w; the epilogue parks the tile's results in the same memory
   constexpr int SLAB_BYTES = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16_t);
   constexpr int OUT_BYTES = tile_out_bytes<BM, BN, OUTMODE>() + tile_slot_bytes<BM, OUTMODE>();
   __shared__ __attribute__((aligned(16))) char smem[SLAB_BYTES > OUT_BYTES ? SLAB_BYTES : OUT_BYTES];      // shared by the two bodies
-  if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);
-  else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem);
+  if (K % BKT == 0) gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, false>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem, gr);
+  else gemm_tile_body<BM, BN, WM, WN, PF, ACT, OUTMODE, true>(a, lda, w, ldw, ep, kv, M, N, K, tiles_m, tiles_n, smem, gr);
 }
 
 template <int BM, int BN, int WM, int WN, int PF, int ACT>
 static void launch_tile_act(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                            const KvScatter& kv, int M, int N, int K) {
+                            const KvScatter& kv, int M, int N, int K, const Grouping& gr) {
   const int tiles_m = da_ceil_div(M, BM), tiles_n = da_ceil_div(N, BN);
   const dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if (ep.accumulate)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 2>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n, gr);
   else if (ep.out_dtype == DA_F32)
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 1>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n, gr);
   else
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, BN, WM, WN, PF, ACT, 0>), grid, block, 0, s, A, lda, W, ldw, ep, kv, M, N, K, tiles_m, tiles_n, gr);
 }
 
 template <int BM, int BN, int WM, int WN, int PF>
 static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W, int ldw, const Epilogue& ep,
-                        const KvScatter& kv, int M, int N, int K) {
+                        const KvScatter& kv, int M, int N, int K, const Grouping& gr = Grouping{nullptr, 0, 0}) {
   switch (ep.act) {
-    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
-    default: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_GELU_TANH: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_TANH>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
+    case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
+    case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
+    case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
+    default: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
   }
 }
 
@@ -780,5 +794,31 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
     else launch_tile<64, 64, 2, 2, 4>(s, A, lda, W, ldw, ep, kv, M, N, K);
   }
   DA_CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}
+
+// out = a @ w[group of the row].T on the block tiles: rows come in groups of `group_rows` (128 or a multiple), group i
+// uses the matrix w + tile_group[i] * group_stride elements ([N, K] each), groups with a negative entry are skipped.
+// The same tiles and the same order of sums as da_gemm_bf16's.
+extern "C" int da_gemm_bf16_grouped(const void* a, int lda, const void* w, int ldw, long group_stride,
+                                    const int* tile_group, int group_rows, void* out, int out_dtype, int ldo, int M,
+                                    int N, int K, void* stream) {
+  DA_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_grouped: bad sizes M=%d N=%d K=%d", M, N, K);
+  DA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && group_stride % 8 == 0,
+             "gemm_bf16_grouped: K, lda, ldw and the stride between matrices must be multiples of 8");
+  DA_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_grouped: operands must be 16-byte aligned");
+  DA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_bf16_grouped: leading sizes too small");
+  DA_REQUIRE(tile_group && group_rows > 0 && group_rows % 128 == 0 && M % group_rows == 0,
+             "gemm_bf16_grouped: %d rows in groups of %d (a multiple of 128 that divides the rows)", M, group_rows);
+  DA_REQUIRE(out_dtype == DA_BF16 || out_dtype == DA_F32, "gemm_bf16_grouped: bad output dtype");
+  if (M == 0) return 0;
+  Epilogue ep{nullptr, 0, DA_ACT_NONE, 0, out, out_dtype, ldo};
+  KvScatter kv{nullptr, nullptr, 0, 0, 0, 0, 0};
+  Grouping gr{tile_group, group_stride, group_rows};
+  hipStream_t s = (hipStream_t)stream;
+  const long tiles128 = (long)da_ceil_div(M, 128) * da_ceil_div(N, 128);
+  if (tiles128 >= 192) launch_tile<128, 128, 4, 2, 2>(s, (const bf16_t*)a, lda, (const bf16_t*)w, ldw, ep, kv, M, N, K, gr);
+  else launch_tile<128, 64, 4, 2, 4>(s, (const bf16_t*)a, lda, (const bf16_t*)w, ldw, ep, kv, M, N, K, gr);
+  DA_CHECK_LAUNCH("gemm_bf16_grouped");
   return 0;
 }

@@ -346,3 +346,27 @@ extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot
   DA_CHECK_LAUNCH("moe_down_mfma");
   return 0;
 }
+
+// rows of a in the order of the slots (zeros for slots that hold no pair): the operand of the grouped block-tile
+// product, 16 bytes a thread
+__global__ void moe_gather_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
+                                  bf16_t* __restrict__ out, int rows, int width8) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)rows * width8) return;
+  const int slot = (int)(i / width8), c = (int)(i % width8) * 8;
+  const int r = row_of_slot[slot];
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (r >= 0) v = *(const uint4*)(a + (size_t)r * lda + c);
+  *(uint4*)(out + (size_t)slot * width8 * 8 + c) = v;
+}
+
+extern "C" int da_moe_gather(const void* a, int lda, const int* row_of_slot, void* out, int rows, int width, void* stream) {
+  DA_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0 && lda % 8 == 0 && lda >= width, "moe_gather: the width must be a multiple of 8");
+  DA_REQUIRE((uintptr_t)a % 16 == 0 && (uintptr_t)out % 16 == 0, "moe_gather: operands must be 16-byte aligned");
+  if (rows == 0) return 0;
+  const long n = (long)rows * (width / 8);
+  hipLaunchKernelGGL(moe_gather_kernel, dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a, lda,
+                     row_of_slot, (bf16_t*)out, rows, width / 8);
+  DA_CHECK_LAUNCH("moe_gather");
+  return 0;
+}

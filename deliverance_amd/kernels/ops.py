@@ -105,6 +105,8 @@ _ARGTYPES = {
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
+    "da_moe_gather": [_VP, _I, _VP, _VP, _I, _I, _VP],
+    "da_gemm_bf16_grouped": [_VP, _I, _VP, _I, ctypes.c_long, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_combine": [_VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _I, _I, _VP],
 }
 _LIB = None
@@ -333,7 +335,8 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------- experts
 MOE_TILE_ROWS = 64       # rows of a tile of the plain grouped products
-MOE_TILE_ROWS_MFMA = 32  # ... of the matrix-core grouped products (csrc/moe.hip)
+MOE_TILE_ROWS_MFMA = 32  # ... of the matrix-core grouped products for few rows an expert (csrc/moe.hip)
+MOE_TILE_ROWS_BLOCK = 128  # ... of the block-tile product with a matrix per group of rows (csrc/gemm_mfma.hip)
 
 
 def moe_slot_space(n_tokens: int, top: int, n_experts: int, tile: int):
@@ -1020,14 +1023,35 @@ def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Te
     N, width = h.shape
     inner = down.shape[2]
     mfma = _moe_mfma_ok(h, gate_up, down)
-    tile = MOE_TILE_ROWS_MFMA if mfma else MOE_TILE_ROWS
+    # Many rows an expert (prompt portions): the rows are gathered expert by expert and go through the block
+    # tiles of the dense products, a matrix per group of 128 rows.  Few (decoding): tiles of 32 rows that
+    # stream each expert's weights once.  The choice reads the step's shape only.
+    block = mfma and N * top >= 64 * n_experts and inner % 8 == 0
+    tile = MOE_TILE_ROWS_BLOCK if block else (MOE_TILE_ROWS_MFMA if mfma else MOE_TILE_ROWS)
     tiles, rows = moe_slot_space(N, top, n_experts, tile)
     ints = ctx.buf("moe_route", N * top + rows + tiles, 1, torch.int32).view(-1)
     slot_of_pair, row_of_slot, tile_expert = ints[:N * top], ints[N * top:N * top + rows], ints[N * top + rows:]
     moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
     mid = ctx.buf("moe_mid", rows, inner, h.dtype)
     pair_out = ctx.buf("moe_out", rows, width, torch.float32)
-    if mfma:
+    if block:
+        _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, 2 * inner, width)
+              and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
+        _dev(h, gate_up, down)
+        hs = ctx.buf("moe_rows", rows, width, h.dtype)
+        gu = ctx.buf("moe_gate_up", rows, 2 * inner, h.dtype)
+        with _timed("experts_gather", 2 * N * top * width * 2, 0):
+            _check(_lib().da_moe_gather(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(hs), rows, width, _stream()))
+        with _timed("experts_gate_up", N * top * (width + 2 * inner) * 2 + _nbytes(gate_up), 4 * N * top * inner * width):
+            _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, 2 * inner * width,
+                                               _ptr(tile_expert), tile, _ptr(gu), BF16, gu.stride(0), rows, 2 * inner, width,
+                                               _stream()))
+        gated_act(gu, mid, act)
+        with _timed("experts_down", N * top * (inner * 2 + width * 4) + _nbytes(down), 2 * N * top * inner * width):
+            _check(_lib().da_gemm_bf16_grouped(_ptr(mid), mid.stride(0), _ptr(down), inner, width * inner,
+                                               _ptr(tile_expert), tile, _ptr(pair_out), F32, pair_out.stride(0), rows, width,
+                                               inner, _stream()))
+    elif mfma:
         _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, 2 * inner, width)
               and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
         _dev(h, gate_up, down)
