@@ -41,6 +41,7 @@
 #ifdef PF_REL
 #define PF_KERNEL attn_prefill_rel_kernel
 #define PF_REL_MAX_DIST 1024       // entries of the bias row that the workgroup keeps in LDS
+#define PF_REL_PAD 96              // a tile's keys reach at most 59 + 35 distances past either end of the row
 #define PF_REL_PARAMS , const float* __restrict__ rel_bias, int n_dist, float t_coef, int t_every
 #define PF_REL_ARGS , rel_bias, n_dist, t_coef, t_every
 #else
@@ -89,7 +90,10 @@ PF_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cac
   bf16_t (*Vs2)[V_TILE] = (bf16_t (*)[V_TILE])(smem + NB * K_TILE * 2);
   __shared__ long long bts[KP == 1 ? PF_BT_MAX : PF_BT_MAX_PHASED];   // a page's place in the cache, in bytes
 #ifdef PF_REL
-  __shared__ float brel[PF_REL_MAX_DIST];       // the head's bias by distance, times log2 e (zeros without a table)
+  // The head's bias by distance, times log2 e (zeros without a table), in descending order of the distance and
+  // with PF_REL_PAD entries beyond both ends (the first and the last value again): a lane's 32 keys of a tile
+  // are then 32 fixed places behind one address, and nothing is clamped per key.
+  __shared__ float brel[PF_REL_MAX_DIST + 2 * PF_REL_PAD];
 #endif
 
   // The workgroups with the most keys (the last rows) are launched first, those of every (sequence, head) pair
@@ -142,7 +146,11 @@ PF_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cac
   const float scale2 = scale * 1.4426950408889634f *
                        (t_every > 0 ? 1.0f + t_coef * logf((float)(((q_ok ? pq : 0) + 1) / t_every + 1)) : 1.0f);
   const int n_rel = rel_bias ? n_dist : 1;
-  for (int i = t; i < n_rel; i += THREADS) brel[i] = rel_bias ? rel_bias[(size_t)h * n_dist + i] * 1.4426950408889634f : 0.f;
+  const int rel_len = n_rel + 2 * PF_REL_PAD;
+  for (int i = t; i < rel_len; i += THREADS) {       // place i holds the distance rel_len - 1 - PF_REL_PAD - i
+    const int dist = rel_len - 1 - PF_REL_PAD - i, dc = dist < 0 ? 0 : (dist < n_rel ? dist : n_rel - 1);
+    brel[i] = rel_bias ? rel_bias[(size_t)h * n_dist + dc] * 1.4426950408889634f : 0.f;
+  }
 #else
   const float scale2 = scale * 1.4426950408889634f;
 #endif
@@ -301,17 +309,17 @@ PF_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cac
       const int d0 = (q_ok ? pq : -(1 << 30)) - kt - 4 * hf;      // pq - key for the lane's first key
       const int e0 = (pq - q_lo) - d0;                             // key - q_lo likewise
       const bool far = kt + PF_BK - 1 <= w_first - (n_rel - 1);    // every key n_rel - 1 or more behind every row
-      const float bfar = brel[n_rel - 1];
+      const float bfar = brel[0];
+      // the lane's key c of the tile lies d0 - c behind its row: place (rel_len - 1 - PF_REL_PAD - d0) + c.  One
+      // clamp a tile keeps rows that do not exist inside the table; rows that do never reach it (see PF_REL_PAD).
+      const int d0c = d0 < 59 - PF_REL_PAD ? 59 - PF_REL_PAD : (d0 > n_rel - 1 + PF_REL_PAD ? n_rel - 1 + PF_REL_PAD : d0);
+      const float* bp = brel + (rel_len - 1 - PF_REL_PAD - d0c);
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int c = ks * 32 + 8 * (r / 4) + (r % 4);
-          float b = bfar;
-          if (!far) {
-            const int dist = d0 - c;
-            b = brel[dist < 0 ? 0 : (dist < n_rel ? dist : n_rel - 1)];
-          }
+          const float b = far ? bfar : bp[c];
           float v = __builtin_fmaf(sc[ks][r], scale2, b);
           if (!whole) {
             const int lo = min(d0 - c, e0 + c);

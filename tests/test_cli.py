@@ -26,6 +26,20 @@ def test_random_then_inspect(tmp_path):
     assert "h.2.mlp.c_fc.weight" in p.stdout and "[96, 200]" in p.stdout
 
 
+def test_random_then_inspect_another_design(tmp_path):
+    """The same commands on a Virudra configuration: the registry picks the design by config.json."""
+    from virudra_models import CONFIG_Y
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(CONFIG_Y))
+    out = tmp_path / "model"
+    p = run("random", "--config", str(cfg), "--seed", "3", "--out", str(out))
+    assert p.returncode == 0, p.stderr
+    p = run("inspect", str(out))
+    assert p.returncode == 0, p.stderr
+    assert "architecture Virudra: 3 layers, width 96, vocabulary 200" in p.stdout and "3 layer calls, 3 cache slots" in p.stdout
+    assert "l0.mlp.e2.down" in p.stdout and "l2.mlp.table" in p.stdout and "l1.mix.rel" in p.stdout and "[32, 2]" in p.stdout
+
+
 def test_help_names_the_reference_options():
     p = run("generate", "--help")
     for opt in ("--model", "--working-dtype", "--max-tokens", "--temperature", "--seed", "--warmup-cases", "--max-cases",
