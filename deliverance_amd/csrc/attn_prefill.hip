@@ -314,20 +314,37 @@ PF_KERNEL(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cac
       // clamp a tile keeps rows that do not exist inside the table; rows that do never reach it (see PF_REL_PAD).
       const int d0c = d0 < 59 - PF_REL_PAD ? 59 - PF_REL_PAD : (d0 > n_rel - 1 + PF_REL_PAD ? n_rel - 1 + PF_REL_PAD : d0);
       const float* bp = brel + (rel_len - 1 - PF_REL_PAD - d0c);
+      // three straight-line forms, chosen by conditions that hold for the whole wavefront
+      if (whole && far) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int c = ks * 32 + 8 * (r / 4) + (r % 4);
-          const float b = far ? bfar : bp[c];
-          float v = __builtin_fmaf(sc[ks][r], scale2, b);
-          if (!whole) {
-            const int lo = min(d0 - c, e0 + c);
-            v += __builtin_bit_cast(float, (lo >> 31) & (int)0xff800000);
+          for (int r = 0; r < 16; ++r) {
+            const float v = __builtin_fmaf(sc[ks][r], scale2, bfar);
+            sc[ks][r] = v;
+            tmax = fmaxf(tmax, v);
           }
-          sc[ks][r] = v;
-          tmax = fmaxf(tmax, v);
-        }
+      } else if (whole) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float v = __builtin_fmaf(sc[ks][r], scale2, bp[ks * 32 + 8 * (r / 4) + (r % 4)]);
+            sc[ks][r] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int c = ks * 32 + 8 * (r / 4) + (r % 4);
+            const int lo = min(d0 - c, e0 + c);
+            const float v = __builtin_fmaf(sc[ks][r], scale2, bp[c]) + __builtin_bit_cast(float, (lo >> 31) & (int)0xff800000);
+            sc[ks][r] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      }
 #else
       if (whole) {
 #pragma unroll
