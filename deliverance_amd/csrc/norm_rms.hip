@@ -39,12 +39,23 @@ rmsnorm_row_kernel(const float* __restrict__ src, const int* __restrict__ rows, 
   const int r = blockIdx.x * (blockDim.x / DA_WAVE) + threadIdx.x / DA_WAVE;
   if (r >= R) return;
   const float* sr = src + (size_t)(rows ? rows[r] : r) * E;
-  float4 v[VPL], xv[VPL];
+  // Up to a width of 1,024 the gains are asked for beside the rows, so that the kernel costs one round trip
+  // to memory and not one per norm; wider rows have no registers to spare for that and read them when needed.
+  constexpr bool EARLY = VPL <= 4;
+  float4 v[VPL], xv[VPL], ga[EARLY ? VPL : 1], gb[EARLY ? VPL : 1];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
     v[i] = *(const float4*)(sr + (c < E ? c : 0));
     if (ADD) xv[i] = *(const float4*)(x + (size_t)r * E + (c < E ? c : 0));
+  }
+  if (EARLY) {
+#pragma unroll
+    for (int i = 0; i < (EARLY ? VPL : 1); ++i) {
+      const int c = (lane + i * DA_WAVE) * 4, cc = c < E ? c : 0;
+      ga[i] = rms_param4(wa, wa_dtype, cc);
+      if (ADD && y) gb[i] = rms_param4(wb, wb_dtype, cc);
+    }
   }
   float q = 0.f;
 #pragma unroll
@@ -56,7 +67,7 @@ rmsnorm_row_kernel(const float* __restrict__ src, const int* __restrict__ rows, 
   for (int i = 0; i < VPL; ++i) {
     const int c = (lane + i * DA_WAVE) * 4;
     if (c < E) {
-      const float4 g = rms_param4(wa, wa_dtype, c);
+      const float4 g = EARLY ? ga[EARLY ? i : 0] : rms_param4(wa, wa_dtype, c);
       float4 o = make_float4(v[i].x * inv * (offset + g.x), v[i].y * inv * (offset + g.y),
                              v[i].z * inv * (offset + g.z), v[i].w * inv * (offset + g.w));
       if (ADD) {
@@ -75,7 +86,7 @@ rmsnorm_row_kernel(const float* __restrict__ src, const int* __restrict__ rows, 
     for (int i = 0; i < VPL; ++i) {
       const int c = (lane + i * DA_WAVE) * 4;
       if (c < E) {
-        const float4 g = rms_param4(wb, wb_dtype, c);
+        const float4 g = EARLY ? gb[EARLY ? i : 0] : rms_param4(wb, wb_dtype, c);
         rms_store4(y, y_dtype, (size_t)r * E + c,
                    make_float4(xv[i].x * inv2 * (offset + g.x), xv[i].y * inv2 * (offset + g.y),
                                xv[i].z * inv2 * (offset + g.z), xv[i].w * inv2 * (offset + g.w)));
