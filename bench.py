@@ -135,7 +135,7 @@ def virudra_config(name, n_positions=1024):
                "mlp": {"kind": "dense", "ff": F} if i % 2 == 0 else
                       {"kind": "moe", "expert": {"ff": F // 2}, "router": {"experts": 8, "top": 2}}}
               for i in range(g["n_layer"])]
-    return {"architecture": "Virudra", "vocab": 50257, "width": E, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    return {"architecture": "Virudra", "vocab": 50257, "width": E, "norm": {"eps": 1e-5}, "logit_softcap": 50.0,
             "layers": layers, "max_positions": n_positions,
             # what decode_run and prefill_run read
             "vocab_size": 50257, "n_positions": n_positions, "n_layer": g["n_layer"], "n_embd": E, "ff": F}

@@ -32,7 +32,7 @@ RUNS = {
                ["tests/test_virudra_gpu.py", "-n", "3", "-k",
                 "(rms_norm_kernels and 64) or (every_edge and bfloat16) or (experts_feed_forward_part and (64-24 or 300) and bfloat16) "
                 "or (gated_feed_forward_part and 64-40) or (attention_with_bias and bfloat16 and 4-2-16-16) or softcap "
-                "or (mixed and Y and bfloat16) or (portions and X and float32 and 31)"],
+                "or (whole_prompts and Z and bfloat16)"],
     "replay": ["tests/test_replay_gpu.py", "-n", "4"] if FULL else
               ["tests/test_replay_gpu.py", "-n", "2", "-k", "(mixed and (A or B) and not 32) or want_subset or errors_leave or first_tokens"],
     # inner sizes of 32 in an engine step: qkv and fc of seed 11 (and, in the full run, proj of seed 5)
