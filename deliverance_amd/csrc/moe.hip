@@ -251,9 +251,8 @@ template <bool GATED>
 __global__ void __launch_bounds__(256)
 moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
                 const int* __restrict__ tile_expert, const bf16_t* __restrict__ w, void* __restrict__ out, int ldo,
-                int K, int F, int act, int n_rows) {
-  // without routing arrays: one matrix and the rows 0 .. n_rows - 1 as they lie (a dense gated feed-forward)
-  const int e = tile_expert ? tile_expert[blockIdx.y] : 0;
+                int K, int F, int act) {
+  const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
   const int fr = lane % 16, fk = (lane / 16) * 8;
@@ -265,7 +264,7 @@ moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ r
   int srow[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    srow[i] = row_of_slot ? row_of_slot[m0 + i * 16 + fr] : (m0 + i * 16 + fr < n_rows ? m0 + i * 16 + fr : -1);
+    srow[i] = row_of_slot[m0 + i * 16 + fr];
     const int r = GATED ? (srow[i] >= 0 ? srow[i] : 0) : m0 + i * 16 + fr;
     ap[i] = a + (size_t)r * lda + fk;
   }
@@ -308,7 +307,7 @@ moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ r
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int row = 4 * (lane / 16) + r;
-      const int used = row_of_slot ? row_of_slot[m0 + i * 16 + row] : (m0 + i * 16 + row < n_rows ? 0 : -1);
+      const int used = row_of_slot[m0 + i * 16 + row];
       if (used < 0 || n0 + fr >= F) continue;
       const size_t o = (size_t)(m0 + i * 16 + row) * ldo + n0 + fr;
       if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(acc[i][0][r], act) * acc[i][GATED ? 1 : 0][r]);
@@ -324,18 +323,14 @@ static int moe_mfma_checks(const void* a, int lda, const void* w, int K, const c
 
 extern "C" int da_moe_tile_rows_mfma() { return MM_ROWS; }
 
-// row_of_slot and tile_expert both null: no routing, w is one matrix [2 F, K] and rows 0 .. n_rows - 1 of a are taken
-// as they lie (T_cap tiles of 32 rows cover them).
 extern "C" int da_moe_gated_mfma(const void* a, int lda, const int* row_of_slot, const int* tile_expert, const void* w,
-                                 void* mid, int ldm, int T_cap, int K, int F, int act, int n_rows, void* stream) {
+                                 void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
   DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_mfma: bad sizes");
-  DA_REQUIRE((row_of_slot == nullptr) == (tile_expert == nullptr), "moe_gated_mfma: both routing arrays, or neither");
-  DA_REQUIRE(row_of_slot || (n_rows >= 0 && n_rows <= T_cap * MM_ROWS), "moe_gated_mfma: %d rows in %d tiles", n_rows, T_cap);
   DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "moe_gated_mfma: unknown activation %d", act);
   if (moe_mfma_checks(a, lda, w, K, "moe_gated_mfma")) return 1;
   if (T_cap == 0) return 0;
   hipLaunchKernelGGL((moe_mfma_kernel<true>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, n_rows);
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act);
   DA_CHECK_LAUNCH("moe_gated_mfma");
   return 0;
 }
@@ -347,7 +342,7 @@ extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot
   if (T_cap == 0) return 0;
   hipLaunchKernelGGL((moe_mfma_kernel<false>), dim3(da_ceil_div(width, MM_COLS), T_cap), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F,
-                     width, 0, 0);
+                     width, 0);
   DA_CHECK_LAUNCH("moe_down_mfma");
   return 0;
 }

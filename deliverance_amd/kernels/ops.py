@@ -103,7 +103,7 @@ _ARGTYPES = {
     "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP],
     "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
-    "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_gather": [_VP, _I, _VP, _VP, _I, _I, _VP],
     "da_gemm_bf16_grouped": [_VP, _I, _VP, _I, ctypes.c_long, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP],
@@ -336,7 +336,6 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 # ------------------------------------------------------------------------------- experts
 MOE_TILE_ROWS = 64       # rows of a tile of the plain grouped products
 MOE_TILE_ROWS_MFMA = 32  # ... of the matrix-core grouped products for few rows an expert (csrc/moe.hip)
-GATED_FUSED_MAX_ROWS = 64   # steps up to which a dense gated feed-forward's first product runs as one fused kernel
 MOE_TILE_ROWS_BLOCK = 128  # ... of the block-tile product with a matrix per group of rows (csrc/gemm_mfma.hip)
 
 
@@ -1006,22 +1005,6 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
 def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
     """mid = act(h @ gate.T) * (h @ up.T) with gate | up as one matrix [2 inner, width]."""
     N, inner = mid.shape
-    # Few rows: one kernel that streams gate and up rows of the same columns side by side and applies the
-    # activation in its epilogue (the experts' kernel without routing); else the tuned product and the
-    # activation as two kernels.
-    if (_MODE == "tuned" and 0 < N <= GATED_FUSED_MAX_ROWS and h.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16
-            and mid.dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and h.stride(0) % 8 == 0 and h.data_ptr() % 16 == 0
-            and gate_up.data_ptr() % 16 == 0 and gate_up.is_contiguous()):
-        _dev(h, gate_up, mid)
-        _rows_2d(h, "h"); _rows_2d(mid, "mid")
-        K = h.shape[1]
-        _need(tuple(gate_up.shape) == (2 * inner, K), "gated_linear: gate|up must be [2 inner, width]")
-        if not (act in ACTIVATIONS):
-            raise KernelError(f"gated_linear: unknown activation {act!r}")
-        with _timed("gated_product_fused", _nbytes(h, gate_up, mid), 4 * N * inner * K):
-            _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), None, None, _ptr(gate_up), _ptr(mid), mid.stride(0),
-                                            -(-N // MOE_TILE_ROWS_MFMA), K, inner, ACTIVATIONS[act], N, _stream()))
-        return mid
     gu = ctx.buf("ff_gate_up", N, 2 * inner, h.dtype)
     linear(h, gate_up, None, gu)
     return gated_act(gu, mid, act)
@@ -1076,7 +1059,7 @@ def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Te
         nb = N * top * (width * 2 + inner * 2) + min(n_experts, N * top) * 2 * inner * width * 2
         with _timed("experts_gated", nb, 4 * N * top * inner * width):
             _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
-                                            _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], 0, _stream()))
+                                            _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], _stream()))
         nb = N * top * (inner * 2 + width * 4) + min(n_experts, N * top) * inner * width * 2
         with _timed("experts_down", nb, 2 * N * top * inner * width):
             _check(_lib().da_moe_down_mfma(_ptr(mid), mid.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(down),
