@@ -273,7 +273,7 @@ def ff_ctx(dtype, tokens):
 
 
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
-@pytest.mark.parametrize("E,F,N", [quick(64, 40, 5), (96, 200, 70)])
+@pytest.mark.parametrize("E,F,N", [quick(64, 40, 5), (80, 104, 40), (96, 200, 70)])
 def test_gated_feed_forward_part(dtype, E, F, N):
     from deliverance_amd.config.specs import GatedFeedForwardSpec
     from deliverance_amd.parts import build_feed_forward
