@@ -455,3 +455,49 @@ def test_greedy_generation_through_the_engine(vmodels, name, dtype):
                 row = m.plain_logits(ids)[-1]
                 assert row[t] >= row.max() - 2 * 6e-2 * float(np.sqrt((row ** 2).mean()))
                 ids.append(t)
+
+
+# ------------------------------------------------------------------------------------------ random configurations
+def random_config(seed):
+    """Sizes drawn at random, among them what the kernels take only on their plain paths: widths that are no
+    multiple of 8 or 4, head sizes that are no multiple of 16, values of another size, bias tables longer than the
+    prefill kernel's copy, one expert, as many experts a token as there are, loops over any range."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *a: a[int(rng.integers(0, len(a)))]
+    width = pick(40, 50, 64, 100, 72, 36)
+    n_layers = int(rng.integers(1, 4))
+    layers = []
+    for _ in range(n_layers):
+        G = pick(1, 2, 3)
+        H = G * pick(1, 2, 3)
+        D = pick(8, 16, 24, 32, 64)
+        Dv = pick(D, D, 8, 40)
+        buckets = pick(2, 4, 5, 9, 16, 30)
+        far = buckets // 2 + pick(1, 3, 20, 200, 1500)
+        mlp = pick(None, "dense", "moe", "moe")
+        if mlp == "dense":
+            mlp = _dense = {"kind": "dense", "ff": pick(24, 40, 100)}
+        elif mlp == "moe":
+            n = pick(1, 2, 5, 9)
+            mlp = {"kind": "moe", "expert": {"ff": pick(8, 20, 32)}, "router": {"experts": n, "top": pick(1, n, max(1, n // 2))}}
+        layers.append({"type": "attention", "mlp": mlp,
+                       "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": Dv, "scale": float(pick(0.1, D ** -0.5, 0.3)),
+                                 "bias_max": far, "bias_buckets": buckets,
+                                 "q_temp": {"coef": float(pick(0.0, 0.25, 1.5)), "every": pick(1, 3, 16, 500)}}})
+    a = int(rng.integers(0, n_layers + 1))
+    b = int(rng.integers(a, n_layers + 1))
+    cfg = {"architecture": "Virudra", "vocab": pick(50, 130, 257), "width": width, "norm": {"eps": float(pick(1e-6, 1e-5, 1e-3))},
+           "logit_softcap": float(pick(5.0, 25.0, 100.0)), "layers": layers}
+    if pick(True, True, False):
+        cfg["loop"] = {"start": a, "stop": b, "times": pick(1, 2, 3)}
+    return cfg
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(tmp_path, seed, dtype):
+    m = make_model(tmp_path / "m", random_config(seed), 100 + seed)
+    ids = m.prompt(45, salt=seed)
+    s = helpers.trace_session(m.folder, dtype, 128, poison_freed=True)
+    check(m, helpers.replay(s, helpers.trace_whole("w", ids)), [("w", ids)], dtype, f"seed {seed} whole")
+    check(m, helpers.replay(s, helpers.trace_portions("p", ids, (5, 2, 17, 1, 1, 9))), [("p", ids)], dtype, f"seed {seed} portions")
