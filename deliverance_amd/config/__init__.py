@@ -2,7 +2,8 @@ from .specs import (AttentionSpec, ConfigError, DenseFeedForwardSpec, LayerCall,
                     ModelConfig, NormSpec, PositionSpec)
 from .gpt2 import Gpt2Config
 from .virudra import VirudraConfig
+from .pedatar import PedatarConfig
 from .engine_config import EngineConfig
 
 __all__ = ["AttentionSpec", "ConfigError", "DenseFeedForwardSpec", "LayerCall", "LayerSpec",
-           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "VirudraConfig", "EngineConfig"]
+           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "VirudraConfig", "PedatarConfig", "EngineConfig"]

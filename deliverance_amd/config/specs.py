@@ -92,11 +92,60 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class RotarySpec:
+    """Pairs of the first ``dims`` entries of a query or key vector are turned by the angle position * speed_i,
+    speed_i = base^(-2i / dims), i = 0 .. dims / 2 - 1; entries behind ``dims`` pass.  ``interleaved``: pair i is
+    (2i, 2i + 1), else (i, i + dims / 2).  (u, v) becomes (u cos a - v sin a, v cos a + u sin a)."""
+    kind: str            # "rotary"
+    dims: int
+    base: float
+    interleaved: bool = True
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are linear maps of one narrow normalised vector a token.
+
+    The mixer's input h goes down to [ query latent (q_rank) | latent (kv_rank) | key piece (rot_dim) ].  Both
+    latents pass a root-mean-square norm with a gain (``norm_eps``).  Queries are ``up_q`` of the query latent:
+    per head ``head_dim`` entries that meet the head's keys ``up_k`` of the latent, and ``rot_dim`` entries that are
+    turned by the position and meet the turned key piece, which all heads share.  Values are ``up_v`` of the latent,
+    ``v_head_dim`` a head.  The cache keeps the latent and the turned key piece, nothing per head."""
+    kind: str            # "latent_attention"
+    width: int
+    n_heads: int
+    head_dim: int        # unrotated entries of a head's queries and keys
+    rot_dim: int         # rotated entries (a head's queries; one shared key piece)
+    v_head_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    rotary: RotarySpec
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class SelectiveScanSpec:
+    """A selective state-space mixer: the input goes up to [ x | z ] of ``inner`` channels each; x passes a causal
+    filter of ``conv_taps`` taps per channel and SiLU; from x come a step size per channel (through ``dt_rank``
+    numbers, a matrix, a bias and softplus) and two vectors B, C of ``state`` entries; per channel c and state
+    index j, S[c, j] <- exp(dt_c A[c, j]) S[c, j] + dt_c x_c B_j with A = -exp(A_log), y_c = sum_j S[c, j] C_j + D_c x_c;
+    the output is the down-projection of y * silu(z).  The state (S and the filter's last inputs) is 32-bit."""
+    kind: str            # "selective_scan"
+    width: int
+    inner: int
+    state: int
+    dt_rank: int
+    conv_taps: int
+
+
+@dataclass(frozen=True)
 class DenseFeedForwardSpec:
     kind: str            # "dense"
     width: int
     inner: int
-    activation: str      # "gelu_new" | "gelu" | "gelu_pytorch_tanh" | "relu" | "silu"
+    activation: str      # "gelu_new" | "gelu" | "gelu_pytorch_tanh" | "relu" | "silu" | "relu2"
     bias: bool = True
 
 
@@ -111,9 +160,14 @@ class GatedFeedForwardSpec:
 
 @dataclass(frozen=True)
 class ExpertsFeedForwardSpec:
-    """``n_experts`` gated feed-forwards of ``inner`` columns, of which every token uses ``top``; the output is
-    the weighted sum of theirs.  ``router == "token_table"``: a table [vocab, top] of integers names each
-    token id's experts (a row's entries differ), each with weight 1 / top."""
+    """``n_experts`` feed-forwards of ``inner`` columns, of which every token uses ``top``; the output is the
+    weighted sum of theirs.  ``router == "token_table"``: a table [vocab, top] of integers names each token id's
+    experts (a row's entries differ), each with weight 1 / top.  ``router == "logistic_top"``: a matrix
+    [n_experts, width] gives 32-bit logits z; the ``top`` experts with the largest logistic(z) are used, with those
+    scores as weights (``renormalize``: divided by their sum).  ``gated``: an expert is down(act(gate h) * (up h)),
+    else down(act(up h)).  ``weight_on``: "output" (weight * expert(h)) or "input" (expert(weight * h)).
+    ``shared_inner`` > 0: one more feed-forward of that many columns, of the ungated form, runs for every token
+    with weight 1 and is added."""
     kind: str            # "experts"
     width: int
     inner: int
@@ -122,6 +176,11 @@ class ExpertsFeedForwardSpec:
     activation: str
     router: str = "token_table"
     vocab_size: int = 0
+    gated: bool = True
+    weight_on: str = "output"
+    renormalize: bool = False
+    shared_inner: int = 0
+    shared_activation: Optional[str] = None
 
 
 @dataclass(frozen=True)

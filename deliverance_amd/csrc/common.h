@@ -16,6 +16,8 @@
 #define DA_ACT_GELU_ERF 2
 #define DA_ACT_RELU 3
 #define DA_ACT_SILU 4
+#define DA_ACT_RELU2 5      // the square of max(x, 0)
+#define DA_ACT_LAST DA_ACT_RELU2
 
 #define DA_WAVE 64
 
@@ -195,6 +197,10 @@ __device__ __forceinline__ float apply_act(float x, int act) {
       return fmaxf(x, 0.0f);
     case DA_ACT_SILU:
       return x / (1.0f + expf(-x));
+    case DA_ACT_RELU2: {
+      const float r = fmaxf(x, 0.0f);
+      return r * r;
+    }
     default:
       return x;
   }

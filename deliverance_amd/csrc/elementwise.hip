@@ -14,7 +14,7 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, int ld, T* __restrict
 
 extern "C" int da_gated_act(const void* gu, int ld, int dtype, void* mid, int ldm, int R, int inner, int act, void* stream) {
   DA_REQUIRE(R >= 0 && inner > 0 && ld >= 2 * inner && ldm >= inner, "gated_act: bad sizes R=%d inner=%d", R, inner);
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gated_act: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gated_act: unknown activation %d", act);
   if (R == 0) return 0;
   const long n = (long)R * inner;
   if (dtype == DA_BF16)

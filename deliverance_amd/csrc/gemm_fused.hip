@@ -399,7 +399,7 @@ static int gemm_bf16_norm(const float* x, const int* rows, const void* g, int g_
   DA_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
              (!b || (uintptr_t)b % 16 == 0), "gemm_bf16_ln: operands must be 16-byte aligned");
   DA_REQUIRE(eps > 0.f, "gemm_bf16_ln: eps must be > 0");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16_ln: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gemm_bf16_ln: unknown activation %d", act);
   if (kv_cache) {
     DA_REQUIRE(out_dtype == DA_BF16 && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N && page > 0,
                "gemm_bf16_ln: the q|k|v columns (%d + 2*%d) must add up to N=%d", q_cols, kv_cols, N);

@@ -394,6 +394,7 @@ static void launch_tile(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
     case DA_ACT_GELU_ERF: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
     case DA_ACT_RELU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
     case DA_ACT_SILU: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
+    case DA_ACT_RELU2: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_RELU2>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
     default: launch_tile_act<BM, BN, WM, WN, PF, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K, gr); break;
   }
 }
@@ -750,7 +751,7 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
   DA_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
   DA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_bf16: leading sizes too small");
   DA_REQUIRE(!accumulate || out_dtype == DA_F32, "gemm_bf16: accumulation needs a 32-bit output");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gemm_bf16: unknown activation %d", act);
   if (kv_cache) {
     DA_REQUIRE(out_dtype == DA_BF16 && !accumulate && q_cols >= 0 && kv_cols == Hkv * D && q_cols + 2 * kv_cols == N &&
                page > 0 && (page & (page - 1)) == 0, "gemm_bf16: the q|k|v columns (%d + 2*%d) must add up to N=%d, the page size a power of two", q_cols, kv_cols, N);
@@ -802,7 +803,7 @@ extern "C" int da_gemm_bf16(const void* a, int lda, const void* w, int ldw, cons
 // The same tiles and the same order of sums as da_gemm_bf16's.
 extern "C" int da_gemm_bf16_grouped(const void* a, int lda, const void* w, int ldw, long group_stride,
                                     const int* tile_group, int group_rows, void* out, int out_dtype, int ldo, int M,
-                                    int N, int K, void* stream) {
+                                    int N, int K, void* stream, int act) {
   DA_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_grouped: bad sizes M=%d N=%d K=%d", M, N, K);
   DA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && group_stride % 8 == 0,
              "gemm_bf16_grouped: K, lda, ldw and the stride between matrices must be multiples of 8");
@@ -811,8 +812,9 @@ extern "C" int da_gemm_bf16_grouped(const void* a, int lda, const void* w, int l
   DA_REQUIRE(tile_group && group_rows > 0 && group_rows % 128 == 0 && M % group_rows == 0,
              "gemm_bf16_grouped: %d rows in groups of %d (a multiple of 128 that divides the rows)", M, group_rows);
   DA_REQUIRE(out_dtype == DA_BF16 || out_dtype == DA_F32, "gemm_bf16_grouped: bad output dtype");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gemm_bf16_grouped: unknown activation %d", act);
   if (M == 0) return 0;
-  Epilogue ep{nullptr, 0, DA_ACT_NONE, 0, out, out_dtype, ldo};
+  Epilogue ep{nullptr, 0, act, 0, out, out_dtype, ldo};
   KvScatter kv{nullptr, nullptr, 0, 0, 0, 0, 0};
   Grouping gr{tile_group, group_stride, group_rows};
   hipStream_t s = (hipStream_t)stream;

@@ -96,7 +96,7 @@ extern "C" int da_gemm_ref(const void* a, int lda, const void* w, int ldw, int i
   DA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_ref: leading sizes too small (lda=%d ldw=%d ldo=%d)",
              lda, ldw, ldo);
   DA_REQUIRE(!accumulate || out_dtype == DA_F32, "gemm_ref: accumulation needs a 32-bit output");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_ref: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gemm_ref: unknown activation %d", act);
   if (M == 0) return 0;
   dim3 grid(da_ceil_div(N, TILE), da_ceil_div(M, TILE));
   if (in_dtype == DA_BF16)

@@ -412,6 +412,7 @@ static void launch_wide(hipStream_t s, const bf16_t* A, int lda, const bf16_t* W
     case DA_ACT_GELU_ERF: launch_wide_act<BM, BN, WM, WN, DA_ACT_GELU_ERF>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
     case DA_ACT_RELU: launch_wide_act<BM, BN, WM, WN, DA_ACT_RELU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
     case DA_ACT_SILU: launch_wide_act<BM, BN, WM, WN, DA_ACT_SILU>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
+    case DA_ACT_RELU2: launch_wide_act<BM, BN, WM, WN, DA_ACT_RELU2>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
     default: launch_wide_act<BM, BN, WM, WN, DA_ACT_NONE>(s, A, lda, W, ldw, ep, kv, M, N, K); break;
   }
 }
@@ -465,7 +466,7 @@ extern "C" int da_gemm_bf16_wide(const void* a, int lda, const void* w, int ldw,
   DA_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldo >= N, "gemm_bf16_wide: leading sizes (lda=%d ldw=%d ldo=%d)", lda, ldw, ldo);
   DA_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_wide: operands must be 16-byte aligned");
   DA_REQUIRE(!accumulate || out_dtype == DA_F32, "gemm_bf16_wide: accumulation needs a 32-bit output");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "gemm_bf16_wide: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "gemm_bf16_wide: unknown activation %d", act);
   DA_REQUIRE(da_gemm_wide_takes(act, accumulate, out_dtype, K),
              "gemm_bf16_wide: K=%d must be a multiple of %d, and an activation goes with a bfloat16 result", K, WD_BK);
   if (kv_cache) {

@@ -83,13 +83,19 @@ extern "C" int da_moe_route(const int* tokens, const int* table, int vocab, cons
 #define MBK 16
 #define MCHUNK 8
 
-// GATED: two products (gate and up rows of the expert's stacked matrix), out = act(g) * u in T;
-// else one product, 32-bit out.  GATHER: row r of the tile is a[row_of_slot[slot]], else a[slot].
-template <typename T, bool GATED>
+// MOE_GATED: two products (gate and up rows of the expert's stacked matrix), out = act(g) * u in T; MOE_UP: one
+// product, out = act(.) in T; MOE_DOWN: one product, 32-bit out.  The first two gather: row r of the tile is
+// a[row_of_slot[slot]] (times slot_scale[slot] when given: the sums are scaled, which is the same number),
+// MOE_DOWN reads a[slot].
+#define MOE_DOWN 0
+#define MOE_GATED 1
+#define MOE_UP 2
+template <typename T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
                        const int* __restrict__ tile_expert, const T* __restrict__ w, void* __restrict__ out, int ldo,
-                       int K, int F, int act) {
+                       int K, int F, int act, const float* __restrict__ slot_scale) {
+  constexpr bool GATED = MODE == MOE_GATED, GATHER = MODE != MOE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   __shared__ float As[MBK][MT + 4];
@@ -110,7 +116,7 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[g][i][j] = part[g][i][j] = 0.f;
-  const int arow = GATED ? srow[lrow] : (srow[lrow] >= 0 ? m0 + lrow : -1);
+  const int arow = GATHER ? srow[lrow] : (srow[lrow] >= 0 ? m0 + lrow : -1);
   int slab = 0;
   for (int k0 = 0; k0 < K; k0 += MBK) {
 #pragma unroll
@@ -162,6 +168,7 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
   for (int i = 0; i < 4; ++i) {
     const int r = ty * 4 + i;
     if (srow[r] < 0) continue;
+    const float sc = (GATHER && slot_scale) ? slot_scale[m0 + r] : 1.0f;      // the row of a times its weight
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
@@ -169,9 +176,11 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
       const size_t o = (size_t)(m0 + r) * ldo + n;
       if (GATED) {
         if (DTypeOf<T>::value == DA_BF16)
-          from_f32(&((T*)out)[o], apply_act_bf16(acc[0][i][j], act) * acc[1][i][j]);
+          from_f32(&((T*)out)[o], apply_act_bf16(sc * acc[0][i][j], act) * (sc * acc[1][i][j]));
         else
-          from_f32(&((T*)out)[o], apply_act(acc[0][i][j], act) * acc[1][i][j]);
+          from_f32(&((T*)out)[o], apply_act(sc * acc[0][i][j], act) * (sc * acc[1][i][j]));
+      } else if (MODE == MOE_UP) {
+        from_f32(&((T*)out)[o], DTypeOf<T>::value == DA_BF16 ? apply_act_bf16(sc * acc[0][i][j], act) : apply_act(sc * acc[0][i][j], act));
       } else {
         ((float*)out)[o] = acc[0][i][j];
       }
@@ -182,15 +191,15 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
 extern "C" int da_moe_gated_ref(const void* a, int lda, int dtype, const int* row_of_slot, const int* tile_expert,
                                 const void* w, void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
   DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_ref: bad sizes");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "moe_gated_ref: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_gated_ref: unknown activation %d", act);
   if (T_cap == 0) return 0;
   dim3 grid(da_ceil_div(F, MT), T_cap);
   if (dtype == DA_BF16)
-    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, true>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
-                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act);
+    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_GATED>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
+                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr);
   else
-    hipLaunchKernelGGL((moe_product_ref_kernel<float, true>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
-                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act);
+    hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_GATED>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
+                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, nullptr);
   DA_CHECK_LAUNCH("moe_gated_ref");
   return 0;
 }
@@ -201,12 +210,84 @@ extern "C" int da_moe_down_ref(const void* mid, int ldm, int dtype, const int* r
   if (T_cap == 0) return 0;
   dim3 grid(da_ceil_div(width, MT), T_cap);
   if (dtype == DA_BF16)
-    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, false>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F, width, 0);
+    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_DOWN>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F, width, 0, nullptr);
   else
-    hipLaunchKernelGGL((moe_product_ref_kernel<float, false>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const float*)mid, ldm, row_of_slot, tile_expert, (const float*)w, out, ldo, F, width, 0);
+    hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_DOWN>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const float*)mid, ldm, row_of_slot, tile_expert, (const float*)w, out, ldo, F, width, 0, nullptr);
   DA_CHECK_LAUNCH("moe_down_ref");
+  return 0;
+}
+
+// mid[slot] = act(scale[slot] * (W_e a[row_of_slot[slot]])): the first product of experts without a gate; w: [experts, F, K]
+extern "C" int da_moe_up_ref(const void* a, int lda, int dtype, const int* row_of_slot, const int* tile_expert,
+                             const void* w, const float* slot_scale, void* mid, int ldm, int T_cap, int K, int F, int act,
+                             void* stream) {
+  DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_up_ref: bad sizes");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_up_ref: unknown activation %d", act);
+  if (T_cap == 0) return 0;
+  dim3 grid(da_ceil_div(F, MT), T_cap);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_UP>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
+                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale);
+  else
+    hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_UP>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
+                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, slot_scale);
+  DA_CHECK_LAUNCH("moe_up_ref");
+  return 0;
+}
+
+// The router of a mixture whose scores are logistic(z): every token's `top` largest (the lower index wins a tie),
+// ids[n, k] and weights[n, k] in descending order of the score.  `renorm`: the weights divided by their sum.
+__global__ void moe_top_logistic_kernel(const float* __restrict__ z, int ldz, int N, int E, int top, int renorm,
+                                        int* __restrict__ ids, float* __restrict__ weights) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  const float* row = z + (size_t)n * ldz;
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bz = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      const float v = row[e];
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= ids[(size_t)n * top + j] == e;
+      if (!taken && (best < 0 || v > bz)) { best = e; bz = v; }
+    }
+    const float sc = 1.0f / (1.0f + expf(-bz));
+    ids[(size_t)n * top + k] = best;
+    weights[(size_t)n * top + k] = sc;
+    sum += sc;
+  }
+  if (renorm)
+    for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] /= sum;
+}
+
+extern "C" int da_moe_top_logistic(const float* z, int ldz, int N, int E, int top, int renorm, int* ids, float* weights,
+                                   void* stream) {
+  DA_REQUIRE(N >= 0 && E > 0 && top > 0 && top <= E && ldz >= E, "moe_top_logistic: bad sizes");
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(moe_top_logistic_kernel, dim3(da_ceil_div(N, 64)), dim3(64), 0, (hipStream_t)stream, z, ldz, N, E, top,
+                     renorm, ids, weights);
+  DA_CHECK_LAUNCH("moe_top_logistic");
+  return 0;
+}
+
+// slot_weight[slot_of_pair[i]] = weights[i]: a pair's weight where its slot's row is
+__global__ void moe_slot_weights_kernel(const int* __restrict__ slot_of_pair, const float* __restrict__ weights, int P,
+                                        float* __restrict__ slot_weight) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  const int slot = slot_of_pair[i];
+  if (slot >= 0) slot_weight[slot] = weights[i];
+}
+
+extern "C" int da_moe_slot_weights(const int* slot_of_pair, const float* weights, int P, float* slot_weight, void* stream) {
+  DA_REQUIRE(P >= 0, "moe_slot_weights: bad size");
+  if (P == 0) return 0;
+  hipLaunchKernelGGL(moe_slot_weights_kernel, dim3(da_ceil_div(P, 256)), dim3(256), 0, (hipStream_t)stream, slot_of_pair,
+                     weights, P, slot_weight);
+  DA_CHECK_LAUNCH("moe_slot_weights");
   return 0;
 }
 
@@ -247,11 +328,12 @@ extern "C" int da_moe_combine(const float* out, int ldo, const int* slot_of_pair
 #define MM_COLS 64
 #define MM_UNROLL 4
 
-template <bool GATED>
+template <int MODE>
 __global__ void __launch_bounds__(256)
 moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
                 const int* __restrict__ tile_expert, const bf16_t* __restrict__ w, void* __restrict__ out, int ldo,
-                int K, int F, int act) {
+                int K, int F, int act, const float* __restrict__ slot_scale) {
+  constexpr bool GATED = MODE == MOE_GATED, GATHER = MODE != MOE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
@@ -265,7 +347,7 @@ moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ r
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     srow[i] = row_of_slot[m0 + i * 16 + fr];
-    const int r = GATED ? (srow[i] >= 0 ? srow[i] : 0) : m0 + i * 16 + fr;
+    const int r = GATHER ? (srow[i] >= 0 ? srow[i] : 0) : m0 + i * 16 + fr;
     ap[i] = a + (size_t)r * lda + fk;
   }
   const int wcol = n0 + fr < F ? n0 + fr : 0;
@@ -310,7 +392,9 @@ moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ r
       const int used = row_of_slot[m0 + i * 16 + row];
       if (used < 0 || n0 + fr >= F) continue;
       const size_t o = (size_t)(m0 + i * 16 + row) * ldo + n0 + fr;
-      if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(acc[i][0][r], act) * acc[i][GATED ? 1 : 0][r]);
+      const float sc = (GATHER && slot_scale) ? slot_scale[m0 + i * 16 + row] : 1.0f;
+      if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(sc * acc[i][0][r], act) * (sc * acc[i][GATED ? 1 : 0][r]));
+      else if (MODE == MOE_UP) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(sc * acc[i][0][r], act));
       else ((float*)out)[o] = acc[i][0][r];
     }
 }
@@ -326,12 +410,24 @@ extern "C" int da_moe_tile_rows_mfma() { return MM_ROWS; }
 extern "C" int da_moe_gated_mfma(const void* a, int lda, const int* row_of_slot, const int* tile_expert, const void* w,
                                  void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
   DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_mfma: bad sizes");
-  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_SILU, "moe_gated_mfma: unknown activation %d", act);
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_gated_mfma: unknown activation %d", act);
   if (moe_mfma_checks(a, lda, w, K, "moe_gated_mfma")) return 1;
   if (T_cap == 0) return 0;
-  hipLaunchKernelGGL((moe_mfma_kernel<true>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act);
+  hipLaunchKernelGGL((moe_mfma_kernel<MOE_GATED>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr);
   DA_CHECK_LAUNCH("moe_gated_mfma");
+  return 0;
+}
+
+extern "C" int da_moe_up_mfma(const void* a, int lda, const int* row_of_slot, const int* tile_expert, const void* w,
+                              const float* slot_scale, void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
+  DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_up_mfma: bad sizes");
+  DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_up_mfma: unknown activation %d", act);
+  if (moe_mfma_checks(a, lda, w, K, "moe_up_mfma")) return 1;
+  if (T_cap == 0) return 0;
+  hipLaunchKernelGGL((moe_mfma_kernel<MOE_UP>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale);
+  DA_CHECK_LAUNCH("moe_up_mfma");
   return 0;
 }
 
@@ -340,9 +436,9 @@ extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot
   DA_REQUIRE(T_cap >= 0 && F > 0 && width > 0 && ldm >= F && ldo >= width, "moe_down_mfma: bad sizes");
   if (moe_mfma_checks(mid, ldm, w, F, "moe_down_mfma")) return 1;
   if (T_cap == 0) return 0;
-  hipLaunchKernelGGL((moe_mfma_kernel<false>), dim3(da_ceil_div(width, MM_COLS), T_cap), dim3(256), 0,
+  hipLaunchKernelGGL((moe_mfma_kernel<MOE_DOWN>), dim3(da_ceil_div(width, MM_COLS), T_cap), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F,
-                     width, 0);
+                     width, 0, nullptr);
   DA_CHECK_LAUNCH("moe_down_mfma");
   return 0;
 }
@@ -350,23 +446,31 @@ extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot
 // rows of a in the order of the slots (zeros for slots that hold no pair): the operand of the grouped block-tile
 // product, 16 bytes a thread
 __global__ void moe_gather_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
-                                  bf16_t* __restrict__ out, int rows, int width8) {
+                                  bf16_t* __restrict__ out, int rows, int width8, const float* __restrict__ slot_scale) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (long)rows * width8) return;
   const int slot = (int)(i / width8), c = (int)(i % width8) * 8;
   const int r = row_of_slot[slot];
   uint4 v = make_uint4(0, 0, 0, 0);
   if (r >= 0) v = *(const uint4*)(a + (size_t)r * lda + c);
+  if (slot_scale && r >= 0) {                     // the row times its pair's weight, rounded once
+    const float sc = slot_scale[slot];
+    uint32_t* w2 = (uint32_t*)&v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w2[e] = pack2_bf16(sc * bf16_to_f32((bf16_t)(w2[e] & 0xffffu)), sc * bf16_to_f32((bf16_t)(w2[e] >> 16)));
+  }
   *(uint4*)(out + (size_t)slot * width8 * 8 + c) = v;
 }
 
-extern "C" int da_moe_gather(const void* a, int lda, const int* row_of_slot, void* out, int rows, int width, void* stream) {
+extern "C" int da_moe_gather(const void* a, int lda, const int* row_of_slot, void* out, int rows, int width, void* stream,
+                             const float* slot_scale) {
   DA_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0 && lda % 8 == 0 && lda >= width, "moe_gather: the width must be a multiple of 8");
   DA_REQUIRE((uintptr_t)a % 16 == 0 && (uintptr_t)out % 16 == 0, "moe_gather: operands must be 16-byte aligned");
   if (rows == 0) return 0;
   const long n = (long)rows * (width / 8);
   hipLaunchKernelGGL(moe_gather_kernel, dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a, lda,
-                     row_of_slot, (bf16_t*)out, rows, width / 8);
+                     row_of_slot, (bf16_t*)out, rows, width / 8, slot_scale);
   DA_CHECK_LAUNCH("moe_gather");
   return 0;
 }

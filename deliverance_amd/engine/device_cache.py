@@ -31,15 +31,18 @@ class DeviceCache:
         for slot in sorted(needs):
             need = needs[slot]
             if isinstance(need, KVNeed):
-                by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window, need.v_head_dim), []).append(slot)
+                by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window, need.v_head_dim,
+                                     bool(getattr(need, "values_in_keys", False))), []).append(slot)
             elif isinstance(need, StateNeed):
                 state_specs.append(StateSpec(slot, need.elems))
                 state_needs[slot] = need
             else:
                 raise TypeError(f"cache slot {slot}: unknown kind of need {need!r}")
-        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w, _), slots in by_shape.items()]
-        # per group: the per-head size of values where it differs from the keys' (None: the same)
-        self.v_head_dims: List[Optional[int]] = [dv if dv != d else None for (_, d, _, dv) in by_shape]
+        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w, _, _), slots in by_shape.items()]
+        # per group: the per-head size of values where it differs from the keys' (None: the same; 0: the values
+        # are read out of the key rows and take no room)
+        self.v_head_dims: List[Optional[int]] = [0 if shared else (dv if dv != d else None)
+                                                 for (_, d, _, dv, shared) in by_shape]
         self.n_pages = -(-max_cached_tokens // page_size)
         self.group_of_slot: Dict[int, int] = {}
         self.kv: Dict[int, torch.Tensor] = {}
@@ -47,7 +50,8 @@ class DeviceCache:
         for g, spec in enumerate(self.groups):
             dv = self.v_head_dims[g]
             # keys and values of one size: [pages, 2, Hkv, page, D]; values of their own size: a page is
-            # Hkv * page * D keys, then Hkv * Dv * page values, [pages, Hkv * page * (D + Dv)]
+            # Hkv * page * D keys, then Hkv * Dv * page values, [pages, Hkv * page * (D + Dv)]; values inside
+            # the keys: rows of Hkv * D entries, token by token, [pages, page * Hkv * D]
             shape = (2, spec.n_kv_heads, page_size, spec.head_dim) if dv is None else \
                 (spec.n_kv_heads * page_size * (spec.head_dim + dv),)
             t = torch.empty((len(spec.slots), self.n_pages, *shape), dtype=dtype, device=self.device)
@@ -82,7 +86,7 @@ class DeviceCache:
 
     def bytes_per_token(self) -> int:
         el = torch.empty((), dtype=self.dtype).element_size()
-        return sum(len(g.slots) * g.n_kv_heads * (g.head_dim + (dv or g.head_dim)) * el
+        return sum(len(g.slots) * g.n_kv_heads * (g.head_dim + (g.head_dim if dv is None else dv)) * el
                    for g, dv in zip(self.groups, self.v_head_dims))
 
     def state_bytes(self) -> int:
@@ -97,7 +101,8 @@ class DeviceCache:
     def tokens_for_budget(needs: Dict[int, object], dtype: torch.dtype, budget_bytes: int, n_state_slots: int = 0) -> int:
         """How many tokens' keys and values fit into ``budget_bytes`` once the state slots are paid for."""
         el = torch.empty((), dtype=dtype).element_size()
-        per_token = sum(n.n_kv_heads * (n.head_dim + (n.v_head_dim or n.head_dim)) * el
+        per_token = sum(n.n_kv_heads * (n.head_dim + (0 if getattr(n, "values_in_keys", False) else
+                                                      (n.v_head_dim or n.head_dim))) * el
                         for n in needs.values() if isinstance(n, KVNeed))
         left = budget_bytes - DeviceCache.state_bytes_for(needs, n_state_slots)
         return max(0, left // max(per_token, 1))

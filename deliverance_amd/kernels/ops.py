@@ -16,7 +16,8 @@ from ..profiler import KernelProfiler
 
 F32, BF16 = 0, 1
 MAX_HEAD_DIM = 256          # what the plain attention kernel takes; the matrix-core kernels: multiples of 16 up to it
-ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4}
+ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4,
+               "relu2": 5}       # relu2: the square of max(x, 0)
 
 
 class KernelError(RuntimeError):
@@ -105,8 +106,19 @@ _ARGTYPES = {
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
-    "da_moe_gather": [_VP, _I, _VP, _VP, _I, _I, _VP],
-    "da_gemm_bf16_grouped": [_VP, _I, _VP, _I, ctypes.c_long, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_gather": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP],
+    "da_gemm_bf16_grouped": [_VP, _I, _VP, _I, ctypes.c_long, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP, _I],
+    "da_moe_up_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_up_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_top_logistic": [_VP, _I, _I, _I, _I, _I, _VP, _VP, _VP],
+    "da_moe_slot_weights": [_VP, _VP, _I, _VP, _VP],
+    "da_rotary": [_VP, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_latent_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP],
+    "da_attn_latent_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_conv_causal": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
+    "da_conv_state_update": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _I, _I, _I, _VP],
+    "da_selective_scan": [_VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _I, _VP, ctypes.c_long, _VP, _VP,
+                          _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP],
     "da_moe_combine": [_VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _I, _I, _VP],
 }
 _LIB = None
@@ -1016,12 +1028,32 @@ def _moe_mfma_ok(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> 
             and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0)
 
 
-def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                    n_experts: int, top: int, weight: float, act: str, x: torch.Tensor, accumulate: bool) -> torch.Tensor:
-    """x (+)= sum_k weight * expert_{table[token, k]}(h): route, two grouped products, combine.  bfloat16 steps
-    run the grouped products on the matrix cores; 32-bit and the reference mode use the plain ones."""
+def moe_top_logistic(z: torch.Tensor, top: int, renorm: bool, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """Every row's ``top`` largest entries of z (32-bit router logits): ids[n, k] and weights[n, k] =
+    logistic(z[n, ids[n, k]]) in descending order (the lower index wins a tie); ``renorm``: divided by their sum."""
+    _dev(z, ids, weights)
+    _rows_2d(z, "z")
+    N, E = z.shape
+    _need(z.dtype == torch.float32, "moe_top_logistic: router logits must be float32")
+    _need(1 <= top <= E, f"moe_top_logistic: top {top} of {E}")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and ids.numel() >= N * top and weights.dtype == torch.float32
+          and weights.is_contiguous() and weights.numel() >= N * top, "moe_top_logistic: ids int32 and weights float32, [N, top]")
+    with _timed("moe_top", N * E * 4 + N * top * 8, N * E * top, "fp32"):
+        _check(_lib().da_moe_top_logistic(_ptr(z), z.stride(0), N, E, top, int(renorm), _ptr(ids), _ptr(weights), _stream()))
+
+
+def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up: torch.Tensor, down: torch.Tensor,
+                    n_experts: int, top: int, weight: float, act: str, x: torch.Tensor, accumulate: bool,
+                    ids: Optional[torch.Tensor] = None, pair_weights: Optional[torch.Tensor] = None,
+                    gated: bool = True, weight_input: bool = False) -> torch.Tensor:
+    """x (+)= sum_k weight_k * expert_k(h) (or, with ``weight_input``, sum_k expert_k(weight_k * h)): route, two
+    grouped products, combine.  The experts of a row come from ``table[token, k]`` or from ``ids[n, k]``; the
+    weights are ``pair_weights[n, k]`` or the one ``weight``.  ``gated``: the first matrix of an expert is gate | up
+    ([2 inner, width]) and its middle is act(gate h) * (up h); else it is [inner, width] and the middle is act(up h).
+    bfloat16 steps run the grouped products on the matrix cores; 32-bit and the reference mode use the plain ones."""
     N, width = h.shape
     inner = down.shape[2]
+    first_rows = (2 if gated else 1) * inner
     mfma = _moe_mfma_ok(h, gate_up, down)
     # Many rows an expert (prompt portions): the rows are gathered expert by expert and go through the block
     # tiles of the dense products, a matrix per group of 128 rows.  Few (decoding): tiles of 32 rows that
@@ -1031,40 +1063,262 @@ def experts_forward(ctx, h: torch.Tensor, table: torch.Tensor, gate_up: torch.Te
     tiles, rows = moe_slot_space(N, top, n_experts, tile)
     ints = ctx.buf("moe_route", N * top + rows + tiles, 1, torch.int32).view(-1)
     slot_of_pair, row_of_slot, tile_expert = ints[:N * top], ints[N * top:N * top + rows], ints[N * top + rows:]
-    moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
+    if ids is None:
+        moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
+    else:
+        moe_route(None, None, ids, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
+    _need(not weight_input or pair_weights is not None, "experts: weights on the input need a weight a pair")
+    slot_scale = None
+    if weight_input:               # a pair's weight where its slot is: the first product scales its rows with it
+        slot_scale = ctx.buf("moe_slot_scale", rows, 1, torch.float32).view(-1)
+        _dev(pair_weights, slot_scale)
+        _need(pair_weights.dtype == torch.float32 and pair_weights.numel() >= N * top, "experts: a float32 weight a pair")
+        _check(_lib().da_moe_slot_weights(_ptr(slot_of_pair), _ptr(pair_weights), N * top, _ptr(slot_scale), _stream()))
     mid = ctx.buf("moe_mid", rows, inner, h.dtype)
     pair_out = ctx.buf("moe_out", rows, width, torch.float32)
+    _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, first_rows, width)
+          and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
+    _dev(h, gate_up, down)
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"experts: unknown activation {act!r}")
     if block:
-        _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, 2 * inner, width)
-              and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
-        _dev(h, gate_up, down)
         hs = ctx.buf("moe_rows", rows, width, h.dtype)
-        gu = ctx.buf("moe_gate_up", rows, 2 * inner, h.dtype)
         with _timed("experts_gather", 2 * N * top * width * 2, 0):
-            _check(_lib().da_moe_gather(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(hs), rows, width, _stream()))
-        with _timed("experts_gate_up", N * top * (width + 2 * inner) * 2 + _nbytes(gate_up), 4 * N * top * inner * width):
-            _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, 2 * inner * width,
-                                               _ptr(tile_expert), tile, _ptr(gu), BF16, gu.stride(0), rows, 2 * inner, width,
-                                               _stream()))
-        gated_act(gu, mid, act)
+            _check(_lib().da_moe_gather(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(hs), rows, width, _stream(),
+                                        _ptr(slot_scale)))
+        if gated:
+            gu = ctx.buf("moe_gate_up", rows, 2 * inner, h.dtype)
+            with _timed("experts_gate_up", N * top * (width + 2 * inner) * 2 + _nbytes(gate_up), 4 * N * top * inner * width):
+                _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, 2 * inner * width,
+                                                   _ptr(tile_expert), tile, _ptr(gu), BF16, gu.stride(0), rows, 2 * inner, width,
+                                                   _stream(), 0))
+            gated_act(gu, mid, act)
+        else:                      # the activation rides in the product's epilogue
+            with _timed("experts_up", N * top * (width + inner) * 2 + _nbytes(gate_up), 2 * N * top * inner * width):
+                _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, inner * width,
+                                                   _ptr(tile_expert), tile, _ptr(mid), BF16, mid.stride(0), rows, inner, width,
+                                                   _stream(), ACTIVATIONS[act]))
         with _timed("experts_down", N * top * (inner * 2 + width * 4) + _nbytes(down), 2 * N * top * inner * width):
             _check(_lib().da_gemm_bf16_grouped(_ptr(mid), mid.stride(0), _ptr(down), inner, width * inner,
                                                _ptr(tile_expert), tile, _ptr(pair_out), F32, pair_out.stride(0), rows, width,
-                                               inner, _stream()))
+                                               inner, _stream(), 0))
     elif mfma:
-        _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, 2 * inner, width)
-              and tuple(down.shape) == (n_experts, width, inner), "experts: stacked weights of the wrong shape")
-        _dev(h, gate_up, down)
         # every expert's weights once (decode: what the step must move), the pairs' rows in and out
-        nb = N * top * (width * 2 + inner * 2) + min(n_experts, N * top) * 2 * inner * width * 2
-        with _timed("experts_gated", nb, 4 * N * top * inner * width):
-            _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
-                                            _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], _stream()))
+        nb = N * top * (width * 2 + inner * 2) + min(n_experts, N * top) * first_rows * width * 2
+        if gated:
+            with _timed("experts_gated", nb, 4 * N * top * inner * width):
+                _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
+                                                _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], _stream()))
+        else:
+            with _timed("experts_up", nb, 2 * N * top * inner * width):
+                _check(_lib().da_moe_up_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
+                                             _ptr(slot_scale), _ptr(mid), mid.stride(0), tiles, width, inner,
+                                             ACTIVATIONS[act], _stream()))
         nb = N * top * (inner * 2 + width * 4) + min(n_experts, N * top) * inner * width * 2
         with _timed("experts_down", nb, 2 * N * top * inner * width):
             _check(_lib().da_moe_down_mfma(_ptr(mid), mid.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(down),
                                            _ptr(pair_out), pair_out.stride(0), tiles, inner, width, _stream()))
     else:
-        moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
+        if gated:
+            moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
+        else:
+            _moe_common(h, row_of_slot, tile_expert, gate_up, tiles, MOE_TILE_ROWS, "moe_up")
+            with _timed("moe_up_plain", _nbytes(h, gate_up, mid), 2 * tiles * MOE_TILE_ROWS * inner * width,
+                        "fp32" if h.dtype == torch.float32 else "bf16"):
+                _check(_lib().da_moe_up_ref(_ptr(h), h.stride(0), _dt(h), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
+                                            _ptr(slot_scale), _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act],
+                                            _stream()))
         moe_down_ref(mid, row_of_slot, tile_expert, down, pair_out, tiles)
-    return moe_combine(pair_out, slot_of_pair, None, weight, top, x, accumulate)
+    if weight_input:               # the weights already sit in the rows
+        return moe_combine(pair_out, slot_of_pair, None, 1.0, top, x, accumulate)
+    return moe_combine(pair_out, slot_of_pair, pair_weights, weight, top, x, accumulate)
+
+
+# ------------------------------------------------------------------------------- rotation, latent attention
+LATENT_MAX_ROW = 1024        # entries of a latent cache row that the attention kernels take (csrc/attn_latent.hip)
+CONV_MAX_TAPS = 16           # taps of a short filter (csrc/ssm.hip)
+SCAN_MAX_STATE = 1024        # state entries a channel of the scan
+
+
+def linear_heads(a: torch.Tensor, a_head_stride: int, a_off: int, w: torch.Tensor, out: torch.Tensor,
+                 out_head_stride: int, out_off: int) -> torch.Tensor:
+    """A product per head: out[:, h * out_head_stride + out_off : .. + n] = a[:, h * a_head_stride + a_off : .. + k]
+    @ w[h].T for the stack w [heads, n, k]; the heads' pieces lie side by side in the rows of a and out."""
+    H, n, k = w.shape
+    _need(a.shape[1] >= (H - 1) * a_head_stride + a_off + k and out.shape[1] >= (H - 1) * out_head_stride + out_off + n,
+          "linear_heads: the heads leave the rows")
+    for h in range(H):
+        linear(a[:, h * a_head_stride + a_off:h * a_head_stride + a_off + k], w[h], None,
+               out[:, h * out_head_stride + out_off:h * out_head_stride + out_off + n])
+    return out
+
+
+def rotary(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, speeds: torch.Tensor, n_heads: int,
+           src_head_stride: int, dst_head_stride: int, width: int, dims: int, interleaved: bool = True) -> torch.Tensor:
+    """dst[n, h, :width] = src[n, h, :width] with the first ``dims`` entries of every head turned in pairs by the angle
+    positions[n] * speeds[i] (float64 [dims / 2]); pairs are (2i, 2i + 1) when ``interleaved``, else (i, i + dims/2).
+    Heads start ``*_head_stride`` entries apart in a row; src and dst may be views into wider rows."""
+    _dev(src, dst, positions, speeds)
+    _rows_2d(src, "src"); _rows_2d(dst, "dst")
+    N = src.shape[0]
+    _need(dst.shape[0] == N and src.dtype == dst.dtype, "rotary: src and dst differ in rows or dtype")
+    _need(positions.dtype == torch.int32 and positions.numel() >= N, "rotary: positions must be int32 [N]")
+    _need(speeds.dtype == torch.float64 and speeds.is_contiguous() and speeds.numel() >= dims // 2,
+          "rotary: speeds must be float64 [dims / 2]")
+    _need(src.shape[1] >= (n_heads - 1) * src_head_stride + width and dst.shape[1] >= (n_heads - 1) * dst_head_stride + width,
+          "rotary: the heads leave the row")
+    with _timed("rotary", 2 * N * n_heads * width * src.element_size(), 3 * N * n_heads * dims, "fp32"):
+        _check(_lib().da_rotary(_ptr(src), src.stride(0), src_head_stride, _ptr(dst), dst.stride(0), dst_head_stride,
+                                _dt(src), _ptr(positions), _ptr(speeds), N, n_heads, width, dims, int(interleaved), _stream()))
+    return dst
+
+
+def latent_cache_row(cache_slot: torch.Tensor, page: int) -> int:
+    """Entries of a row of a latent cache slot [pages, page * D]."""
+    return cache_slot[0].numel() // page
+
+
+def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_gain: Optional[torch.Tensor],
+                   kv_gain: torch.Tensor, eps: float, positions: torch.Tensor, slot_map: Optional[torch.Tensor],
+                   speeds: torch.Tensor, dims: int, interleaved: bool, cq: Optional[torch.Tensor],
+                   cache_slot: torch.Tensor, page: int) -> None:
+    """From rows [ query latent (q_rank) | latent (kv_rank) | key piece (rot_dim) ] of ``down``: cq = rms(query
+    latent) * q_gain; the cache row slot_map[n] = [ rms(latent) * kv_gain | the key piece turned by the position ]."""
+    _dev(down, q_gain, kv_gain, positions, slot_map, speeds, cq, cache_slot)
+    _rows_2d(down, "down")
+    N = down.shape[0]
+    _need(down.shape[1] >= q_rank + kv_rank + rot_dim, "latent_prepare: rows shorter than the three pieces")
+    _need(cache_slot.is_contiguous() and latent_cache_row(cache_slot, page) == kv_rank + rot_dim,
+          "latent_prepare: a row of the cache slot does not hold latent + key piece")
+    _need(kv_gain.numel() == kv_rank and (q_rank == 0 or (q_gain is not None and q_gain.numel() == q_rank and cq is not None)),
+          "latent_prepare: gains differ from the ranks")
+    if cq is not None:
+        _rows_2d(cq, "cq")
+        _need(cq.shape[0] >= N and cq.shape[1] >= q_rank and cq.dtype == cache_slot.dtype, "latent_prepare: cq [N, q_rank] of the cache's dtype")
+    _need(positions.dtype == torch.int32 and positions.numel() >= N and (slot_map is None or (slot_map.dtype == torch.int32 and slot_map.numel() >= N)),
+          "latent_prepare: positions and slot_map must be int32 [N]")
+    _need(speeds.dtype == torch.float64 and speeds.is_contiguous() and speeds.numel() >= dims // 2, "latent_prepare: speeds float64 [dims / 2]")
+    with _timed("latent_prepare", N * (q_rank + kv_rank + rot_dim) * (down.element_size() + cache_slot.element_size()), 6 * N * (q_rank + kv_rank + rot_dim), "fp32"):
+        _check(_lib().da_latent_prepare(_ptr(down), _dt(down), down.stride(0), q_rank, kv_rank, rot_dim, _ptr(q_gain),
+                                        _dt(q_gain) if q_gain is not None else 0, _ptr(kv_gain), _dt(kv_gain), float(eps),
+                                        _ptr(positions), _ptr(slot_map), _ptr(speeds), dims, int(interleaved), _ptr(cq),
+                                        cq.stride(0) if cq is not None else 0, _ptr(cache_slot), _dt(cache_slot), page, N,
+                                        _stream()))
+
+
+def attention_latent_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
+                         positions: torch.Tensor, n_heads: int, row_dim: int, v_dim: int, page: int, scale: float,
+                         window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+    """Plain attention over a latent cache: q [N, Hq * row_dim] (the key maps folded in), out [N, Hq * v_dim] = the
+    weighted sums of the rows' first v_dim entries."""
+    _dev(q, cache_slot, block_table, seq_of_token, positions, out)
+    _rows_2d(q, "q"); _rows_2d(out, "out")
+    N = q.shape[0]
+    _need(cache_slot.is_contiguous() and latent_cache_row(cache_slot, page) == row_dim, "attention_latent: the cache rows differ from q's")
+    _need(q.shape[1] == n_heads * row_dim and out.shape[1] == n_heads * v_dim and out.shape[0] == N and v_dim <= row_dim,
+          "attention_latent: q must be [N, Hq*D] and out [N, Hq*Dv]")
+    _need(q.dtype == cache_slot.dtype == out.dtype, "attention_latent: q, cache and out must share a dtype")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "attention_latent: block_table must be contiguous int32 [S, max_blocks]")
+    _need(seq_of_token.dtype == torch.int32 and positions.dtype == torch.int32 and seq_of_token.numel() >= N
+          and positions.numel() >= N, "attention_latent: ids must be int32, one a row")
+    _check(_lib().da_attn_latent_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table), block_table.shape[1],
+                                     _ptr(seq_of_token), _ptr(positions), N, n_heads, row_dim, v_dim, page, float(scale),
+                                     int(window or 0), _ptr(out), out.stride(0), _stream()))
+    return out
+
+
+def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, row_dim: int,
+                           v_dim: int, scale: float, window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+    """Attention of every row of the step over its sequence's latent rows."""
+    bt = ctx.block_tables[group]
+    page = ctx.cache.page_size
+    el = cache_slot.element_size()
+    lens, starts = ctx.seq_lens_host, ctx.q_start_host        # for the profiler's cost model only
+
+    def cost():
+        if not KernelProfiler.enabled or not lens:
+            return 0, 0
+        keys = pairs = 0
+        for s_ in range(ctx.n_seqs):
+            t = starts[s_ + 1] - starts[s_]
+            n = lens[s_]
+            keys += n
+            pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
+        return keys * row_dim * el + ctx.n_tokens * n_heads * (row_dim + v_dim) * el, 2 * pairs * n_heads * (row_dim + v_dim)
+
+    with _timed("attention_latent_plain", *cost(), "fp32" if q.dtype == torch.float32 else "bf16"):
+        return attention_latent_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, row_dim, v_dim, page,
+                                    scale, window, out)
+
+
+# ------------------------------------------------------------------------------- short filter and scan
+def _state_args(state: torch.Tensor, name: str):
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous(), f"{name}: the state must be contiguous float32 [slots, row]")
+    return state.stride(0)
+
+
+def conv_causal(ctx, x: torch.Tensor, state: torch.Tensor, conv_off: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                act: Optional[str], y: torch.Tensor) -> torch.Tensor:
+    """y[n, c] = act(bias[c] + sum_k weight[c, k] * x[n - (K - 1 - k), c]) within each sequence of the step; rows before
+    the step's portion are the K - 1 inputs that ``state[slot, conv_off:]`` keeps ([K - 1, C], oldest first)."""
+    _dev(x, state, weight, bias, y)
+    _rows_2d(x, "x"); _rows_2d(y, "y")
+    N, C = y.shape
+    K = weight.shape[1]
+    ld = _state_args(state, "conv_causal")
+    _need(x.shape[0] == N and x.shape[1] >= C and x.dtype == y.dtype, "conv_causal: x and y differ")
+    _need(weight.is_contiguous() and tuple(weight.shape) == (C, K) and (bias is None or bias.numel() == C), "conv_causal: weight [C, K], bias [C]")
+    _need(ld >= conv_off + (K - 1) * C, "conv_causal: the state row is too short")
+    if not (act in ACTIVATIONS):
+        raise KernelError(f"conv_causal: unknown activation {act!r}")
+    with _timed("conv_causal", N * C * (x.element_size() * 2), 2 * N * C * K, "fp32"):
+        _check(_lib().da_conv_causal(_ptr(x), _dt(x), x.stride(0), _ptr(state), ld, conv_off, _ptr(ctx.state_slots),
+                                     _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(weight), _dt(weight), _ptr(bias),
+                                     _dt(bias) if bias is not None else 0, ACTIVATIONS[act], _ptr(y), y.stride(0), N, C, K,
+                                     _stream()))
+    return y
+
+
+def conv_state_update(ctx, x: torch.Tensor, state: torch.Tensor, conv_off: int, channels: int, taps: int) -> None:
+    """After the step, ``state[slot, conv_off:]`` holds each sequence's last taps - 1 inputs."""
+    _dev(x, state)
+    _rows_2d(x, "x")
+    ld = _state_args(state, "conv_state_update")
+    _need(x.shape[1] >= channels and ld >= conv_off + (taps - 1) * channels, "conv_state_update: sizes differ")
+    _check(_lib().da_conv_state_update(_ptr(x), _dt(x), x.stride(0), _ptr(state), ld, conv_off, _ptr(ctx.state_slots),
+                                       _ptr(ctx.q_start), ctx.n_seqs, channels, taps, _stream()))
+
+
+SCAN_CHUNK = 64               # tokens of a chunk when a long portion's scan is cut up
+SCAN_CHUNK_FROM = 256         # portions from this length on are cut up
+
+
+def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, z: torch.Tensor,
+                   a_log: torch.Tensor, d: Optional[torch.Tensor], state: torch.Tensor, y: torch.Tensor, n_state: int) -> torch.Tensor:
+    """The scan of a selective state-space mixer over every sequence of the step (see csrc/ssm.hip); the state
+    [slots, >= inner * n_state] is read at each portion's start and written at its end.  Steps whose longest portion
+    has ``SCAN_CHUNK_FROM`` tokens or more are cut into chunks of ``SCAN_CHUNK`` that run side by side."""
+    _dev(x, raw_dt, bc, z, a_log, d, state, y)
+    for t_, nm in ((x, "x"), (raw_dt, "raw_dt"), (bc, "bc"), (z, "z"), (y, "y")):
+        _rows_2d(t_, nm)
+    N, inner = y.shape
+    ld = _state_args(state, "selective_scan")
+    _need(x.shape[0] == N and raw_dt.shape[0] == N and bc.shape[0] == N and z.shape[0] == N, "selective_scan: rows differ")
+    _need(raw_dt.dtype == torch.float32 and x.dtype == y.dtype == bc.dtype == z.dtype, "selective_scan: step sizes in float32, the rest of one dtype")
+    _need(a_log.is_contiguous() and tuple(a_log.shape) == (inner, n_state) and (d is None or d.numel() == inner), "selective_scan: A [inner, state], D [inner]")
+    chunk = max_chunks = 0
+    cs = cd = None
+    if ctx.max_query_len >= SCAN_CHUNK_FROM:
+        chunk = SCAN_CHUNK
+        max_chunks = -(-ctx.max_query_len // chunk)
+        cs = ctx.buf("scan_chunk_state", ctx.n_seqs * max_chunks, inner * n_state, torch.float32)
+        cd = ctx.buf("scan_chunk_dt", ctx.n_seqs * max_chunks, inner, torch.float32)
+    with _timed("selective_scan", N * inner * (x.element_size() * 3 + 4) + N * 2 * n_state * x.element_size(),
+                N * inner * n_state * 6 * (2 if chunk else 1), "fp32"):
+        _check(_lib().da_selective_scan(_ptr(x), _dt(x), x.stride(0), _ptr(raw_dt), raw_dt.stride(0), _ptr(bc), bc.stride(0),
+                                        b_off, c_off, _ptr(z), z.stride(0), _ptr(a_log), _dt(a_log), _ptr(d),
+                                        _dt(d) if d is not None else 0, _ptr(state), ld, _ptr(ctx.state_slots), _ptr(ctx.q_start),
+                                        _ptr(y), y.stride(0), ctx.n_seqs, inner, n_state, chunk, max_chunks, _ptr(cs), _ptr(cd),
+                                        _stream()))
+    return y

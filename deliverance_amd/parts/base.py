@@ -35,11 +35,14 @@ import torch
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Pages of keys (``head_dim`` a head) and values (``v_head_dim`` a head; None: the keys' size)."""
+    """Pages of keys (``head_dim`` a head) and values (``v_head_dim`` a head; None: the keys' size).
+    ``values_in_keys``: nothing is kept for the values, they are the first ``v_head_dim`` entries of the key rows
+    (a page is then ``n_kv_heads * page`` rows of ``head_dim`` entries, token by token)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)

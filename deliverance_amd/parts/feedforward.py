@@ -72,42 +72,77 @@ class GatedFeedForward(FeedForward):
 
 
 class ExpertsFeedForward(FeedForward):
-    """A mixture of gated experts.  The router says which ``top`` experts a token uses and with what weights;
-    ``token_table``: row ``token id`` of an integer table names them, each with weight 1 / top.  The step's
-    (token, choice) pairs are laid out expert by expert on the device (``ops.moe_route``), two grouped
-    products run over that layout, and the pairs' results are added up per token.  Nothing is read back to the
-    host, so a step can be recorded."""
+    """A mixture of experts (``ExpertsFeedForwardSpec``).  The router says which ``top`` experts a token uses and
+    with what weights.  ``token_table``: row ``token id`` of an integer table names them, each with weight 1 / top.
+    ``logistic_top``: 32-bit logits from a matrix; the ``top`` largest logistic scores, which are the weights.
+    The step's (token, choice) pairs are laid out expert by expert on the device (``ops.moe_route``), two grouped
+    products run over that layout, and the pairs' results are added up per token; a weight on the input scales
+    the pair's row in the first product.  A shared expert, if any, runs as a dense feed-forward for every token.
+    Nothing is read back to the host, so a step can be recorded."""
     graph_safe = True
     can_store = True
 
     def __init__(self, spec, params, dtype, device):
         self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
         self.n_experts, self.top, self.router = spec.n_experts, spec.top, spec.router
+        self.gated = bool(getattr(spec, "gated", True))
+        self.weight_on = getattr(spec, "weight_on", "output")
+        self.renormalize = bool(getattr(spec, "renormalize", False))
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}")
-        if self.router != "token_table":
-            raise ValueError(f"unknown router {self.router!r}; known: 'token_table'")
+        if self.router not in ("token_table", "logistic_top"):
+            raise ValueError(f"unknown router {self.router!r}; known: 'token_table', 'logistic_top'")
+        if self.weight_on not in ("output", "input"):
+            raise ValueError(f"a pair's weight goes on the 'output' or the 'input', not {self.weight_on!r}")
         if not (1 <= self.top <= self.n_experts):
             raise ValueError(f"top {self.top} of {self.n_experts} experts")
-        self.gate_up_weight = to_matrix(params["gate_up_weight"], dtype, device)       # [experts, 2 inner, width]
+        first_rows = (2 if self.gated else 1) * self.inner
+        # [experts, 2 inner | inner, width]: gate | up, or up alone
+        self.gate_up_weight = to_matrix(params["gate_up_weight" if self.gated else "up_weight"], dtype, device)
         self.down_weight = to_matrix(params["down_weight"], dtype, device)             # [experts, width, inner]
-        if tuple(self.gate_up_weight.shape) != (self.n_experts, 2 * self.inner, self.width):
-            raise ValueError(f"experts' gate|up weights are {list(self.gate_up_weight.shape)}, expected "
-                             f"{[self.n_experts, 2 * self.inner, self.width]}")
+        if tuple(self.gate_up_weight.shape) != (self.n_experts, first_rows, self.width):
+            raise ValueError(f"experts' first weights are {list(self.gate_up_weight.shape)}, expected "
+                             f"{[self.n_experts, first_rows, self.width]}")
         if tuple(self.down_weight.shape) != (self.n_experts, self.width, self.inner):
             raise ValueError(f"experts' down weights are {list(self.down_weight.shape)}, expected "
                              f"{[self.n_experts, self.width, self.inner]}")
-        table = params["table"]
-        if table.dim() != 2 or table.shape[1] != self.top or (spec.vocab_size and table.shape[0] != spec.vocab_size):
-            raise ValueError(f"expert table is {list(table.shape)}, expected {[spec.vocab_size or 'vocab', self.top]}")
-        if table.dtype not in (torch.int32, torch.int64) or int(table.min()) < 0 or int(table.max()) >= self.n_experts:
-            raise ValueError(f"expert table must hold integers in 0..{self.n_experts - 1}")
-        self.table = table.to(device=device, dtype=torch.int32).contiguous()
+        self.table = self.router_weight = None
+        if self.router == "token_table":
+            table = params["table"]
+            if table.dim() != 2 or table.shape[1] != self.top or (spec.vocab_size and table.shape[0] != spec.vocab_size):
+                raise ValueError(f"expert table is {list(table.shape)}, expected {[spec.vocab_size or 'vocab', self.top]}")
+            if table.dtype not in (torch.int32, torch.int64) or int(table.min()) < 0 or int(table.max()) >= self.n_experts:
+                raise ValueError(f"expert table must hold integers in 0..{self.n_experts - 1}")
+            self.table = table.to(device=device, dtype=torch.int32).contiguous()
+            if self.weight_on != "output":
+                raise ValueError("a table router gives no weight to put on the input")
+        else:
+            self.router_weight = to_matrix(params["router_weight"], dtype, device)     # [experts, width]
+            if tuple(self.router_weight.shape) != (self.n_experts, self.width):
+                raise ValueError(f"router weight is {list(self.router_weight.shape)}, expected {[self.n_experts, self.width]}")
         self.weight = 1.0 / self.top
+        self.shared = None
+        if getattr(spec, "shared_inner", 0):
+            from ..config.specs import DenseFeedForwardSpec
+            self.shared = DenseFeedForward(
+                DenseFeedForwardSpec("dense", self.width, spec.shared_inner, spec.shared_activation or self.activation,
+                                     bias=False),
+                {"fc_weight": params["shared_up_weight"], "proj_weight": params["shared_down_weight"]}, dtype, device)
 
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
+        ids = weights = None
+        if self.router_weight is not None:
+            N = h.shape[0]
+            z = ctx.buf("moe_logits", N, self.n_experts, torch.float32)      # 32-bit sums of the products
+            ops.linear(h, self.router_weight, None, z)
+            ids = ctx.buf("moe_ids", N, self.top, torch.int32)
+            weights = ctx.buf("moe_weights", N, self.top, torch.float32)
+            ops.moe_top_logistic(z, self.top, self.renormalize, ids, weights)
         ops.experts_forward(ctx, h, self.table, self.gate_up_weight, self.down_weight, self.n_experts, self.top,
-                            self.weight, self.activation, x, accumulate=ctx.part_accumulate)
+                            self.weight, self.activation, x, accumulate=ctx.part_accumulate, ids=ids,
+                            pair_weights=weights, gated=self.gated, weight_input=self.weight_on == "input")
+        if self.shared is not None:
+            self.shared.forward(ctx, h, x)
 
 
 register_feed_forward("gated", GatedFeedForward)

@@ -24,3 +24,35 @@ class NoPositions(PositionEncoding):
 
 register_position("learned", LearnedPositions)
 register_position("none", NoPositions)
+
+
+class RotaryPositions(PositionEncoding):
+    """Pairs of a vector's first ``dims`` entries turned by position * base^(-2i / dims) (``RotarySpec``).  The
+    speeds are worked out once in double precision; the kernel takes the sine and cosine of the double angle."""
+
+    def __init__(self, spec, params=None, dtype=None, device=None):
+        import torch
+        self.dims, self.base, self.interleaved = int(spec.dims), float(spec.base), bool(spec.interleaved)
+        if self.dims < 0 or self.dims % 2 != 0:
+            raise ValueError(f"{self.dims} turned entries: an even number is needed")
+        if not (self.base > 0.0):
+            raise ValueError(f"rotation base {self.base} must be positive")
+        speeds = [self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
+        self.speeds = torch.tensor(speeds or [0.0], dtype=torch.float64, device=device)
+
+    def apply(self, ctx, src, dst, n_heads: int, src_head_stride: int, dst_head_stride: int, width: int):
+        """dst[n, h, :width] = turned src[n, h, :width]; heads lie ``*_head_stride`` entries apart in the rows of
+        src and dst (views into wider rows are fine, and src may be dst)."""
+        from ..kernels import ops
+        return ops.rotary(src, dst, ctx.positions, self.speeds, n_heads, src_head_stride, dst_head_stride, width,
+                          self.dims, self.interleaved)
+
+    def apply_qk(self, ctx, qkv, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+        """Queries and keys of a fused q | k | v row, in place."""
+        q = qkv[:, :n_heads * head_dim]
+        k = qkv[:, n_heads * head_dim:(n_heads + n_kv_heads) * head_dim]
+        self.apply(ctx, q, q, n_heads, head_dim, head_dim, head_dim)
+        self.apply(ctx, k, k, n_kv_heads, head_dim, head_dim, head_dim)
+
+
+register_position("rotary", RotaryPositions)

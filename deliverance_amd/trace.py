@@ -31,7 +31,7 @@ class TraceSession:
 
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
                  poison_freed: bool = False, kernels: str = "tuned", use_graphs: bool = False, sample: bool = False,
-                 native_step: bool = True):
+                 native_step: bool = True, state_slots: int = 4):
         import torch
         from . import models  # noqa: F401  (registers the architectures)
         from .config.engine_config import KERNEL_MODES
@@ -44,7 +44,7 @@ class TraceSession:
         # A request's count is rounded up to a multiple of 64, so max_tokens / page_size pages
         # hold every live request whatever its length.
         self.cache = DeviceCache(self.model.cache_needs(), tdtype, device, page_size, max(max_tokens, 64),
-                                 n_state_slots=8, poison_freed=poison_freed)
+                                 n_state_slots=state_slots, poison_freed=poison_freed)
         self.native_step = native_step
         self.runner = self._make_runner(use_graphs, kernels)
         self.sample = sample or use_graphs
@@ -100,6 +100,8 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page: 16, 32 or 64")
+    ap.add_argument("--state-slots", type=int, default=4,
+                    help="requests that can be live at once in a model whose mixers keep a state (default 4)")
     ap.add_argument("--kernels", choices=["tuned", "reference"], default="tuned",
                     help="bfloat16 only: the serving kernels (default) or the plain kernels")
     args = ap.parse_args(argv)
@@ -117,7 +119,8 @@ def main(argv=None) -> int:
         say("no GPU is visible; trace_run drives the GPU engine and has no other path")
         return 3
     say(f"loading {args.model} as {args.dtype}")
-    session = TraceSession(args.model, args.dtype, args.max_tokens, args.page_size, kernels=args.kernels)
+    session = TraceSession(args.model, args.dtype, args.max_tokens, args.page_size, kernels=args.kernels,
+                           state_slots=args.state_slots)
     os.makedirs(args.out, exist_ok=True)
     say("ready")
     for line in sys.stdin:
