@@ -1,0 +1,214 @@
+// Latent attention on the matrix cores (bfloat16): prompt portions and single decoded tokens in one form.
+//
+// All heads of a token read the same cache rows, so the query rows of a workgroup are (token, head) pairs of one
+// sequence: 64 of them, 16 a wavefront, which for decoding is up to 64 heads of one token.  The rows of a tile of
+// 32 cached tokens go from memory into LDS once, row-major for the scores S = Q' K^T and, their first R entries,
+// dimension-major for O = P V (the matrix cores contract over 8 consecutive entries of a lane, which are entries of
+// a row for the scores and tokens for the weighted sums).  MFMA 16x16x32: a lane's fragment is 8 consecutive k of
+// row (or column) lane % 16, k starting at 8 (lane / 16); result r of a lane is row 4 (lane / 16) + r, column
+// lane % 16.  The softmax runs over a wavefront's own 16 rows in 32-bit; the weights pass through LDS to become
+// the first operand of the second product.  The next tile's rows are asked for before this tile's arithmetic.
+// Tiles are walked from the first visible key in steps of 32, so the order of a row's sums depends on the row's
+// own sequence only.
+#include "gemm_common.h"
+
+#define LM_ROWS 64            // query rows a workgroup
+#define LM_KEYS 32            // cached tokens a tile
+#define LM_PAD 8
+
+template <int DB, int RB>     // DB: blocks of 32 entries of a cache row (padded), RB: blocks of 16 entries of R
+__global__ void __launch_bounds__(256)
+attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
+                        const int* __restrict__ block_table, int max_blocks, const int* __restrict__ q_start,
+                        const int* __restrict__ seq_lens, int H, int D, int R, int page, float scale_log2e, int window,
+                        bf16_t* __restrict__ out, int out_ld) {
+  constexpr int D32 = DB * 32;
+  constexpr int ldk = D32 + LM_PAD;                   // entries of a row of the key tile
+  constexpr int ldv = LM_KEYS + LM_PAD;               // entries of a row of the value tile (one entry of R)
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[LM_KEYS * ldk];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * RB * ldv];
+  __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * ldv];
+
+  const int s = blockIdx.y;
+  const int first = q_start[s], T = q_start[s + 1] - first;
+  const int row0 = blockIdx.x * LM_ROWS;
+  if (row0 >= T * H) return;
+  const int len = seq_lens[s];                        // the sequence's length after this step
+  const int past = len - T;                           // position of the portion's first token
+  const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
+  const int fr = lane % 16, fg = lane / 16;
+  const int* bt = block_table + (size_t)s * max_blocks;
+
+  // this lane's fragment row, and the four rows whose results it holds
+  const int arow = row0 + wave * 16 + fr;
+  const bool arow_ok = arow < T * H;
+  const bf16_t* qp = q + (size_t)(first + (arow_ok ? arow / H : 0)) * q_ld + (size_t)(arow_ok ? arow % H : 0) * D + fg * 8;
+  uint4 qf[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int d = i * 32 + fg * 8;
+    qf[i] = (arow_ok && d < D) ? load16(qp + i * 32) : make_uint4(0, 0, 0, 0);
+  }
+  int pos[4];                                         // positions of the rows whose results this lane holds (-1: none)
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = row0 + wave * 16 + 4 * fg + r;
+    pos[r] = row < T * H ? past + row / H : -1;
+  }
+  // the keys this workgroup walks: from the first one its first row sees to the last one its last row sees
+  const int last_row = (row0 + LM_ROWS < T * H ? row0 + LM_ROWS : T * H) - 1;
+  const int p_first = past + row0 / H, p_last = past + last_row / H;
+  const int key_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+
+  floatx4 o[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m[4], l[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { m[r] = -INFINITY; l[r] = 0.f; }
+
+  // zero the padding entries of the key tile once (entries D .. D32 of every row)
+  for (int i = t; i < LM_KEYS * (D32 - D); i += 256) Ks[(i / (D32 - D)) * ldk + D + i % (D32 - D)] = 0;
+  // ... and the rows of the value tile behind R, up to a whole block of 16
+  for (int i = t; i < ((R + 15) / 16 * 16 - R) * ldv; i += 256) Vs[R * ldv + i] = 0;
+
+  const int chunks = D / 8;                           // 16-byte pieces of a cache row
+  const int n_pieces = LM_KEYS * chunks;
+  constexpr int PER = (LM_KEYS * DB * 4 + 255) / 256; // pieces a thread carries
+  uint4 stage[PER];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int pc = t + i * 256;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (pc < n_pieces) {
+        const int key = k0 + pc / chunks;
+        const int pg = key <= p_last ? bt[key / page] : -1;       // rows nobody wrote (or gave back) read as zeros
+        if (pg >= 0) v = load16(cache + ((size_t)pg * page + key % page) * D + (pc % chunks) * 8);
+      }
+      stage[i] = v;
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int pc = t + i * 256;
+      if (pc < n_pieces) {
+        const int kk = pc / chunks, d = (pc % chunks) * 8;
+        *(uint4*)(Ks + kk * ldk + d) = stage[i];
+        if (d < R) {
+          const bf16_t* e = (const bf16_t*)&stage[i];
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (d + j < R) Vs[(d + j) * ldv + kk] = e[j];
+        }
+      }
+    }
+  };
+
+  fetch(key_lo);
+  for (int k0 = key_lo; k0 <= p_last; k0 += LM_KEYS) {
+    __syncthreads();                                  // the tile before has been read by everyone
+    park();
+    __syncthreads();
+    if (k0 + LM_KEYS <= p_last) fetch(k0 + LM_KEYS);
+    // ---- scores of this wavefront's 16 rows against the tile's 32 tokens
+    floatx4 sc[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      sc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kp = Ks + (b * 16 + fr) * ldk + fg * 8;
+#pragma unroll
+      for (int i = 0; i < DB; ++i) {
+        if (i * 32 < D) {
+          const uint4 kf = *(const uint4*)(kp + i * 32);
+          sc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, qf[i]), __builtin_bit_cast(bf16x8_t, kf),
+                                                          sc[b], 0, 0, 0);
+        }
+      }
+    }
+    // ---- the softmax's running maximum and sum, per row, in 32-bit
+    float alpha[4];
+    bf16_t* pw = Ps + wave * 16 * ldv;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float v[2];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int key = k0 + b * 16 + fr;
+        const bool seen = key <= pos[r] && (window <= 0 || key > pos[r] - window);
+        v[b] = seen ? sc[b][r] * scale_log2e : -INFINITY;
+        mx = fmaxf(mx, v[b]);
+      }
+      mx = fmaxf(mx, dpp_move<0xB1, 0xF>(mx, mx));
+      mx = fmaxf(mx, dpp_move<0x4E, 0xF>(mx, mx));
+      mx = fmaxf(mx, dpp_move<0x141, 0xF>(mx, mx));
+      mx = fmaxf(mx, dpp_move<0x140, 0xF>(mx, mx));
+      const float m_new = fmaxf(m[r], mx);
+      const bool none = m_new == -INFINITY;
+      alpha[r] = none ? 1.f : __builtin_amdgcn_exp2f(m[r] - m_new);
+      float sum = 0.f;
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const float e = none ? 0.f : __builtin_amdgcn_exp2f(v[b] - m_new);
+        const bf16_t eb = f32_to_bf16(e);
+        pw[(4 * fg + r) * ldv + b * 16 + fr] = eb;
+        sum += bf16_to_f32(eb);                        // the sum of what the second product really uses
+      }
+      sum = group_sum<16>(sum);
+      l[r] = l[r] * alpha[r] + sum;
+      m[r] = m_new;
+    }
+    // (the weights were written and are read by this wavefront only; LDS operations of a wavefront stay in order)
+    const uint4 pf = *(const uint4*)(pw + fr * ldv + fg * 8);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      if (i * 16 < R) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[i][r] *= alpha[r];
+        const uint4 vf = *(const uint4*)(Vs + (i * 16 + fr) * ldv + fg * 8);
+        o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, pf), __builtin_bit_cast(bf16x8_t, vf), o[i],
+                                                       0, 0, 0);
+      }
+    }
+  }
+  // ---- out[token, head, :R] = O / l
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = row0 + wave * 16 + 4 * fg + r;
+    if (row >= T * H) continue;
+    const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
+    bf16_t* op = out + (size_t)(first + row / H) * out_ld + (size_t)(row % H) * R;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+      if (i * 16 + fr < R) op[i * 16 + fr] = f32_to_bf16(o[i][r] * inv);
+  }
+}
+
+// Whether the matrix-core form takes these sizes: rows of whole 16-byte pieces, up to the largest form's.
+extern "C" int da_attn_latent_mfma_takes(int D, int R) {
+  return D % 8 == 0 && R >= 1 && R <= D && D <= 576 && R <= 512;
+}
+
+extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
+                                   const int* q_start, const int* seq_lens, int S, int max_query_len, int H, int D, int R,
+                                   int page, float scale, int window, void* out, int out_ld, void* stream) {
+  DA_REQUIRE(S >= 0 && H > 0 && page > 0 && max_blocks > 0 && max_query_len > 0 && window >= 0, "attn_latent_mfma: bad sizes");
+  DA_REQUIRE(da_attn_latent_mfma_takes(D, R), "attn_latent_mfma: rows of %d entries with %d of them values are not taken", D, R);
+  DA_REQUIRE(q_ld >= H * D && out_ld >= H * R && q_ld % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)cache % 16 == 0,
+             "attn_latent_mfma: q must hold H * D entries a row in 16-byte pieces");
+  if (S == 0) return 0;
+  const dim3 grid(da_ceil_div((long)max_query_len * H, LM_ROWS), S), block(256);
+  const float sl2 = scale * 1.4426950408889634f;
+  hipStream_t st = (hipStream_t)stream;
+#define DA_LM_GO(DB, RB)                                                                                                  \
+  hipLaunchKernelGGL((attn_latent_mfma_kernel<DB, RB>), grid, block, 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache,   \
+                     block_table, max_blocks, q_start, seq_lens, H, D, R, page, sl2, window, (bf16_t*)out, out_ld)
+  if (D <= 128 && R <= 128) DA_LM_GO(4, 8);
+  else if (D <= 256 && R <= 256) DA_LM_GO(8, 16);
+  else DA_LM_GO(18, 32);
+#undef DA_LM_GO
+  DA_CHECK_LAUNCH("attn_latent_mfma");
+  return 0;
+}

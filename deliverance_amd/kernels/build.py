@@ -31,7 +31,8 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
 # products) keep them in ordinary vector registers; the default puts them into accumulation
 # registers and moves every value out and in again.
 EXTRA_FLAGS = {"attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-               "attn_prefill_rel.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+               "attn_prefill_rel.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+               "attn_latent_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _lib = None
 

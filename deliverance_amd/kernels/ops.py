@@ -115,6 +115,10 @@ _ARGTYPES = {
     "da_rotary": [_VP, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_latent_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP],
     "da_attn_latent_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_latent_mfma": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_latent_mfma_takes": [_I, _I],
+    "da_gemm_heads": [_VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
+    "da_gemm_heads_takes": [_I, _I, _I, _I],
     "da_conv_causal": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
     "da_conv_state_update": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _I, _I, _I, _VP],
     "da_selective_scan": [_VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _I, _VP, ctypes.c_long, _VP, _VP,
@@ -1144,9 +1148,19 @@ def linear_heads(a: torch.Tensor, a_head_stride: int, a_off: int, w: torch.Tenso
                  out_head_stride: int, out_off: int) -> torch.Tensor:
     """A product per head: out[:, h * out_head_stride + out_off : .. + n] = a[:, h * a_head_stride + a_off : .. + k]
     @ w[h].T for the stack w [heads, n, k]; the heads' pieces lie side by side in the rows of a and out."""
+    _rows_2d(a, "a"); _rows_2d(out, "out")
     H, n, k = w.shape
-    _need(a.shape[1] >= (H - 1) * a_head_stride + a_off + k and out.shape[1] >= (H - 1) * out_head_stride + out_off + n,
-          "linear_heads: the heads leave the rows")
+    M = a.shape[0]
+    _need(a.shape[1] >= (H - 1) * a_head_stride + a_off + k and out.shape[1] >= (H - 1) * out_head_stride + out_off + n
+          and out.shape[0] == M, "linear_heads: the heads leave the rows")
+    if (_MODE == "tuned" and a.dtype == w.dtype == out.dtype == torch.bfloat16 and w.is_contiguous()
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and bool(_lib().da_gemm_heads_takes(a.stride(0), a_head_stride, a_off, k))):
+        _dev(a, w, out)
+        with _timed("product_heads", _nbytes(w) + M * H * (n + k) * 2, 2 * M * H * n * k):
+            _check(_lib().da_gemm_heads(_ptr(a), a.stride(0), a_head_stride, a_off, _ptr(w), _ptr(out), out.stride(0),
+                                        out_head_stride, out_off, M, H, n, k, _stream()))
+        return out
     for h in range(H):
         linear(a[:, h * a_head_stride + a_off:h * a_head_stride + a_off + k], w[h], None,
                out[:, h * out_head_stride + out_off:h * out_head_stride + out_off + n])
@@ -1247,6 +1261,22 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
             pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
         return keys * row_dim * el + ctx.n_tokens * n_heads * (row_dim + v_dim) * el, 2 * pairs * n_heads * (row_dim + v_dim)
 
+    if (_MODE == "tuned" and q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
+            and bool(_lib().da_attn_latent_mfma_takes(row_dim, v_dim))):
+        # prompt portions and decoded tokens alike: the query rows of a workgroup are (token, head) pairs
+        _dev(q, cache_slot, bt, out)
+        _rows_2d(q, "q"); _rows_2d(out, "out")
+        _need(cache_slot.is_contiguous() and cache_slot.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+              and latent_cache_row(cache_slot, page) == row_dim, "attention_latent: a bfloat16 cache of rows like q's")
+        _need(q.shape[1] == n_heads * row_dim and out.shape[1] == n_heads * v_dim and out.shape[0] == q.shape[0],
+              "attention_latent: q must be [N, Hq*D] and out [N, Hq*Dv]")
+        _need(bt.dtype == torch.int32 and bt.dim() == 2 and bt.is_contiguous() and bt.shape[0] >= ctx.n_seqs,
+              "attention_latent: block_table must be contiguous int32 [S, max_blocks]")
+        with _timed("attention_latent", *cost()):
+            _check(_lib().da_attn_latent_mfma(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(bt), bt.shape[1], _ptr(ctx.q_start),
+                                              _ptr(ctx.seq_lens), ctx.n_seqs, ctx.max_query_len, n_heads, row_dim, v_dim, page,
+                                              float(scale), int(window or 0), _ptr(out), out.stride(0), _stream()))
+        return out
     with _timed("attention_latent_plain", *cost(), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_latent_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, row_dim, v_dim, page,
                                     scale, window, out)

@@ -88,6 +88,9 @@ class Block:
                                                    else fused(ctx, norm, x, into=into)), part=self.feed_forward,
                        h_ready=h_ff)
             if ctx.debug_hook is not None:
+                chosen = getattr(self.feed_forward, "last_choice", None)
+                if chosen is not None:             # a routed feed-forward: the experts of every row, [N, top]
+                    ctx.emit(call.layer, "expert_choice", chosen)
                 ctx.emit(call.layer, "post_ff_residual", x)
         if self.post_block_norm is not None:                # the stream itself, normalised in place
             ops.copy_rows(self.post_block_norm.forward(ctx, x, out_name="post_norm", out_dtype=torch.float32), x)

@@ -121,6 +121,7 @@ class ExpertsFeedForward(FeedForward):
             if tuple(self.router_weight.shape) != (self.n_experts, self.width):
                 raise ValueError(f"router weight is {list(self.router_weight.shape)}, expected {[self.n_experts, self.width]}")
         self.weight = 1.0 / self.top
+        self.last_choice = None
         self.shared = None
         if getattr(spec, "shared_inner", 0):
             from ..config.specs import DenseFeedForwardSpec
@@ -138,6 +139,7 @@ class ExpertsFeedForward(FeedForward):
             ids = ctx.buf("moe_ids", N, self.top, torch.int32)
             weights = ctx.buf("moe_weights", N, self.top, torch.float32)
             ops.moe_top_logistic(z, self.top, self.renormalize, ids, weights)
+        self.last_choice = ids if ctx.debug_hook is not None else None      # handed to the layer debug hook
         ops.experts_forward(ctx, h, self.table, self.gate_up_weight, self.down_weight, self.n_experts, self.top,
                             self.weight, self.activation, x, accumulate=ctx.part_accumulate, ids=ids,
                             pair_weights=weights, gated=self.gated, weight_input=self.weight_on == "input")

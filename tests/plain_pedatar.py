@@ -131,14 +131,30 @@ def small_ff(W, p, h):
     return squared_ramp(h @ W[p + "up"].T) @ W[p + "down"].T
 
 
-def routed_ff(W, p, mlp, h):
+class FarChoice(AssertionError):
+    """A choice of experts that was handed in ranks far below the ones this implementation makes."""
+
+
+def routed_ff(W, p, mlp, h, given=None, slack=0.0):
     """Every token's ``top`` best experts by logistic(router h); an expert sees the token times its score; a
-    shared expert sees every token as it is."""
+    shared expert sees every token as it is.  ``given[t]`` (optional) are experts that someone else chose for
+    token t: they are used instead of the best ones, provided that each of them lies within ``slack`` (a fraction
+    of the largest router logit's size) of the last place among the best; else FarChoice is raised.  A reduced
+    number format may rank two experts of nearly equal score the other way round, and everything behind such a
+    choice can only be compared when both sides make the same one."""
     n, top = mlp["router"]["experts"], mlp["router"]["top"]
-    score = logistic(h @ W[p + "mlp.router"].T)                          # [T, n]
+    z = h @ W[p + "mlp.router"].T
+    score = logistic(z)                                                  # [T, n]
     out = np.zeros_like(h)
     for t in range(h.shape[0]):
         best = np.argsort(-score[t], kind="stable")[:top]
+        if given is not None and set(int(e) for e in given[t]) != set(int(e) for e in best):
+            theirs = [int(e) for e in given[t]]
+            edge = z[t, best[-1]]
+            if len(set(theirs)) != top or any(z[t, e] < edge - slack * np.abs(z[t]).max() for e in theirs):
+                raise FarChoice(f"{p} token {t}: experts {sorted(theirs)} were chosen, the best are {sorted(int(e) for e in best)} "
+                                f"(router logits {np.round(z[t], 4).tolist()})")
+            best = theirs
         for e in best:
             out[t] += small_ff(W, f"{p}mlp.e{int(e)}.", score[t, e] * h[t][None, :])[0]
     if mlp.get("shared") is not None:
@@ -162,13 +178,14 @@ def layer_runs(cfg):
         yield L, f"l{L.get('weights_of', i)}."
 
 
-def forward(cfg, W, ids, with_layers=False, with_margins=False):
+def forward(cfg, W, ids, with_layers=False, with_margins=False, routes=None, slack=0.0):
     """Logits [T, V] of one whole sequence; with_layers: also the stream after every layer [runs, T, E];
-    with_margins: also the smallest router margin met."""
+    with_margins: also the smallest router margin met.  ``routes[run][t]``: experts chosen elsewhere for token t in
+    the run-th layer (see routed_ff)."""
     eps = cfg["norm"]["eps"]
     x = W["embed"][np.asarray(ids, dtype=np.int64)] * cfg["embedding"]["scale"]
     after, margin = [], np.inf
-    for L, p in layer_runs(cfg):
+    for run, (L, p) in enumerate(layer_runs(cfg)):
         h = unit_rms(x, W[p + "norm1"], eps)
         if L["type"] == "latent_attention":
             x = x + latent_attention(W, p, L["mixer"], h, eps)
@@ -180,7 +197,7 @@ def forward(cfg, W, ids, with_layers=False, with_margins=False):
             h = unit_rms(x, W[p + "norm2"], eps)
             if with_margins:
                 margin = min(margin, float(router_margin(W, p, L["mlp"], h).min()))
-            x = x + routed_ff(W, p, L["mlp"], h)
+            x = x + routed_ff(W, p, L["mlp"], h, None if routes is None else routes.get(run), slack)
         after.append(x.copy())
     logits = unit_rms(x, W["final.norm"], eps) @ W["head"].T
     out = (logits,)
