@@ -17,7 +17,8 @@ its fraction of the roofline; `--no-extra` leaves those two out.  Prints ONE JSO
 `--design virudra` measures another design beside GPT-2 at equal sizes instead (width, heads, head size, layers,
 vocabulary, feed-forward parameters that a token uses): decode at batch 1, 8 and 64 and the prefill of 2 x 1,024
 tokens for both, at the layer sizes of GPT-2 124M and 355M, one JSON line; with `--profile-stages` also both
-models' kernel tables (stderr).
+models' kernel tables (stderr).  `--design pedatar` does the same for a third design beside Virudra (the closest
+of the engine's models to it).
 """
 import argparse
 import json
@@ -160,7 +161,119 @@ def virudra_step_flops(c, seq_lens_new):
     return gemm + attn
 
 
+def pedatar_config(name, n_positions=1024):
+    """A Pedatar of GPT-2 ``name``'s sizes: as many layers, latent attention and selective scans in turn.  Attention:
+    GPT-2's heads with 64 query entries each (48 unrotated, 16 rotated) and values of 64, a query latent of half the
+    width, a latent of a quarter of the width beside a key piece of 16.  Scan: twice the width of channels, 16 state
+    entries, width / 16 step-size numbers, 4 taps.  Feed-forward: 8 experts of the width's size (2 a token) and a
+    shared one of twice the width, which is what GPT-2's two matrices hold for a token."""
+    g = MODELS[name]
+    E, H = g["n_embd"], g["n_head"]
+    att = {"heads": H, "dim": 48, "rot_dim": 16, "vdim": 64, "q_rank": E // 2, "kv_rank": E // 4, "scale": 64 ** -0.5,
+           "rot": {"base": 10000.0, "dims": 16}}
+    scan = {"inner": 2 * E, "state": 16, "dt_rank": E // 16, "conv": 4}
+    mlp = {"kind": "moe", "expert": {"ff": E}, "router": {"experts": 8, "top": 2}, "shared": {"ff": 2 * E}}
+    layers = [{"type": "latent_attention", "mixer": att, "mlp": mlp} if i % 2 == 0 else {"type": "mamba1", "mixer": scan, "mlp": mlp}
+              for i in range(g["n_layer"])]
+    return {"architecture": "Pedatar", "vocab": 50257, "width": E, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "layers": layers, "max_positions": n_positions,
+            # what decode_run and prefill_run read
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": g["n_layer"], "n_embd": E}
+
+
+def _pedatar_layer_params(c, L, experts_used):
+    E = c["width"]
+    m = L["mixer"]
+    if L["type"] == "latent_attention":
+        H, qd = m["heads"], m["dim"] + m["rot_dim"]
+        n = E * (m["q_rank"] + m["kv_rank"] + m["rot_dim"]) + m["q_rank"] * H * qd + m["kv_rank"] * H * (m["dim"] + m["vdim"]) + H * m["vdim"] * E
+    else:
+        I = m["inner"]
+        n = 2 * I * E + I * (m["dt_rank"] + 2 * m["state"]) + m["dt_rank"] * I + I * m["state"] + I * E
+    f = L["mlp"]
+    return n + 2 * E * (experts_used * f["expert"]["ff"] + f["shared"]["ff"]) + f["router"]["experts"] * E
+
+
+def pedatar_step_bytes(c, el, batch, ctx_mean):
+    """What a decode step must read: every matrix once (of the experts as many as ``batch`` tokens can choose), the
+    live requests' latent rows, and the scans' states (read and written, 32-bit)."""
+    n, extra = c["vocab"] * c["width"], 0
+    for L in c["layers"]:
+        f = L["mlp"]["router"]
+        n += _pedatar_layer_params(c, L, min(f["experts"], f["top"] * batch))
+        m = L["mixer"]
+        if L["type"] == "latent_attention":
+            extra += batch * ctx_mean * (m["kv_rank"] + m["rot_dim"]) * el
+        else:
+            extra += batch * 2 * 4 * m["inner"] * (m["state"] + m["conv"] - 1)
+    return n * el + extra
+
+
+def pedatar_step_flops(c, seq_lens_new):
+    """Matrix-product flops of a step (the parameters a token uses, twice), the folded attention's two products over
+    rows of latent + key piece and of latent entries, and the scan's six operations a state entry."""
+    n = sum(seq_lens_new)
+    fl = 2 * len(seq_lens_new) * c["width"] * c["vocab"]
+    for L in c["layers"]:
+        fl += 2 * n * _pedatar_layer_params(c, L, L["mlp"]["router"]["top"])
+        m = L["mixer"]
+        if L["type"] == "latent_attention":
+            pairs = sum(sum(i + 1 for i in range(t)) for t in seq_lens_new)
+            fl += 2 * pairs * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"])
+        else:
+            fl += 6 * n * m["inner"] * m["state"]
+    return fl
+
+
 def design_compare(args):
+    """Decode and prefill of another design beside its like at equal sizes; one JSON line."""
+    if args.design == "pedatar":
+        return pedatar_compare(args)
+    return virudra_compare(args)
+
+
+def pedatar_compare(args):
+    """Decode and prefill of Pedatar beside Virudra (the closest of the engine's models: root-mean-square norms, no
+    position table, mixtures of experts) at the layer sizes of GPT-2 124M and 355M; one JSON line."""
+    import numpy as np
+    el, dkey = 2, "bf16"
+    out = {"metric": "decode tok/s at batch 8 of Pedatar at GPT-2 124M layer sizes (beside Virudra at the same sizes: see points)",
+           "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": dkey, "steps": args.steps, "warmup": args.warmup,
+           "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", "points": {}, "points_frac": {}}
+    for size in ("124m", "355m"):
+        for design in ("virudra", "pedatar"):
+            rng = np.random.default_rng(0)
+            cfg = virudra_config(size) if design == "virudra" else pedatar_config(size)
+            model = engine_from_gpu_weights(cfg, "bfloat16", 64, kernels=args.kernels)
+            key = f"{design}_{size}"
+            for b in (1, 8, 64):
+                steps = min(args.steps, 128)
+                d, cm = decode_run(model, cfg, rng, b, args.prompt_len, steps, 8)
+                out["points"][f"{key}_decode_b{b}"] = round(b * steps / d, 1)
+                if design == "virudra":
+                    nb = virudra_weight_bytes(cfg, el, b) + b * cm * 2 * cfg["n_embd"] * el * cfg["n_layer"]
+                else:
+                    nb = pedatar_step_bytes(cfg, el, b, cm)
+                out["points_frac"][f"{key}_decode_b{b}"] = round(nb / (d / steps) / 1e9 / HBM_GBS, 4)
+            fl = virudra_step_flops(cfg, [1024, 1024]) if design == "virudra" else pedatar_step_flops(cfg, [1024, 1024])
+            pf = prefill_run(model, cfg, rng, dkey, flops=fl)
+            out["points"][f"{key}_prefill_2048"] = pf["value"]
+            out["points_frac"][f"{key}_prefill_2048"] = pf["frac"]
+            if args.profile_stages:
+                print(f"==== {key}", file=sys.stderr)
+                kernel_table(model, cfg, rng, args.batch, args.prompt_len)
+            del model
+    out["value"] = out["points"]["pedatar_124m_decode_b8"]
+    out["config"] = {"model": "pedatar beside virudra at gpt2-124m and gpt2-355m layer sizes", "global_batch": 8,
+                     "prompt_len": args.prompt_len,
+                     "pedatar": "latent attention (48 + 16 query entries a head, values 64, query latent width / 2, latent width / 4 "
+                                "+ key piece 16) and scans (2 x width channels, 16 state entries, 4 taps) in turn; 8 experts of the "
+                                "width's size (2 a token) beside a shared one of twice the width", "parallelism": "single-gpu"}
+    print(json.dumps(out))
+    return 0
+
+
+def virudra_compare(args):
     """Decode and prefill of Virudra beside GPT-2 at equal sizes; one JSON line."""
     import numpy as np
     el, dkey = 2, "bf16"
@@ -322,9 +435,10 @@ def main():
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
                          "requests out of the cache and back, which the line reports as preemptions)")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra"],
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra", "pedatar"],
                     help="virudra: that design beside GPT-2 at equal sizes (decode at batch 1, 8, 64 and the prefill of 2,048 "
-                         "tokens, at 124M and 355M layer sizes) instead of the default workload")
+                         "tokens, at 124M and 355M layer sizes) instead of the default workload; pedatar: that design beside "
+                         "Virudra, likewise")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="mixed: only the mixed workload, on --model (64 requests with prompts of 16 to 895 tokens arrive at "
                          "once, prompt portions of 512 tokens run beside the decoding of the others, 128 new tokens each)")
@@ -336,7 +450,7 @@ def main():
     import numpy as np
     from deliverance_amd.random_model import random_model
 
-    if args.design == "virudra":
+    if args.design in ("virudra", "pedatar"):
         return design_compare(args)
     cfg = model_config(args.model, args.layers, args.n_positions)
     full_layers = MODELS[args.model]["n_layer"]

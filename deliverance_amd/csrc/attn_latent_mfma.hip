@@ -21,7 +21,7 @@ __global__ void __launch_bounds__(256)
 attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                         const int* __restrict__ block_table, int max_blocks, const int* __restrict__ q_start,
                         const int* __restrict__ seq_lens, int H, int D, int R, int page, float scale_log2e, int window,
-                        bf16_t* __restrict__ out, int out_ld) {
+                        bf16_t* __restrict__ out, int out_ld, int seq0, int n_splits, float* __restrict__ partial) {
   constexpr int D32 = DB * 32;
   constexpr int ldk = D32 + LM_PAD;                   // entries of a row of the key tile
   constexpr int ldv = LM_KEYS + LM_PAD;               // entries of a row of the value tile (one entry of R)
@@ -29,7 +29,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * RB * ldv];
   __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * ldv];
 
-  const int s = blockIdx.y;
+  const int s = seq0 + blockIdx.y;
   const int first = q_start[s], T = q_start[s + 1] - first;
   const int row0 = blockIdx.x * LM_ROWS;
   if (row0 >= T * H) return;
@@ -73,45 +73,55 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   for (int i = t; i < ((R + 15) / 16 * 16 - R) * ldv; i += 256) Vs[R * ldv + i] = 0;
 
   const int chunks = D / 8;                           // 16-byte pieces of a cache row
-  const int n_pieces = LM_KEYS * chunks;
-  constexpr int PER = (LM_KEYS * DB * 4 + 255) / 256; // pieces a thread carries
-  uint4 stage[PER];
+  const int n_units = (LM_KEYS / 2) * chunks;         // a unit: the same piece of two neighbouring tokens
+  constexpr int PER = ((LM_KEYS / 2) * DB * 4 + 255) / 256;
+  uint4 stage[PER][2];
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int pc = t + i * 256;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (pc < n_pieces) {
-        const int key = k0 + pc / chunks;
-        const int pg = key <= p_last ? bt[key / page] : -1;       // rows nobody wrote (or gave back) read as zeros
-        if (pg >= 0) v = load16(cache + ((size_t)pg * page + key % page) * D + (pc % chunks) * 8);
+      const int u = t + i * 256;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (u < n_units) {
+          const int key = k0 + 2 * (u / chunks) + e;
+          const int pg = key <= p_last ? bt[key / page] : -1;     // rows nobody wrote (or gave back) read as zeros
+          if (pg >= 0) v = load16(cache + ((size_t)pg * page + key % page) * D + (u % chunks) * 8);
+        }
+        stage[i][e] = v;
       }
-      stage[i] = v;
     }
   };
   auto park = [&]() {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int pc = t + i * 256;
-      if (pc < n_pieces) {
-        const int kk = pc / chunks, d = (pc % chunks) * 8;
-        *(uint4*)(Ks + kk * ldk + d) = stage[i];
-        if (d < R) {
-          const bf16_t* e = (const bf16_t*)&stage[i];
+      const int u = t + i * 256;
+      if (u < n_units) {
+        const int kk = 2 * (u / chunks), d = (u % chunks) * 8;
+        *(uint4*)(Ks + kk * ldk + d) = stage[i][0];
+        *(uint4*)(Ks + (kk + 1) * ldk + d) = stage[i][1];
+        if (d < R) {                                  // dimension-major: the two tokens' entries side by side, one word
+          const bf16_t* e0 = (const bf16_t*)&stage[i][0];
+          const bf16_t* e1 = (const bf16_t*)&stage[i][1];
 #pragma unroll
           for (int j = 0; j < 8; ++j)
-            if (d + j < R) Vs[(d + j) * ldv + kk] = e[j];
+            if (d + j < R) *(uint32_t*)(Vs + (d + j) * ldv + kk) = (uint32_t)e0[j] | ((uint32_t)e1[j] << 16);
         }
       }
     }
   };
 
-  fetch(key_lo);
-  for (int k0 = key_lo; k0 <= p_last; k0 += LM_KEYS) {
+  // the tiles of this workgroup: all of them, or its share when several workgroups split a block's keys
+  const int n_tiles = (p_last - key_lo) / LM_KEYS + 1;
+  const int share = (n_tiles + n_splits - 1) / n_splits;
+  const int k_begin = key_lo + (int)blockIdx.z * share * LM_KEYS;
+  const int k_stop = (k_begin + share * LM_KEYS < p_last + 1) ? k_begin + share * LM_KEYS : p_last + 1;
+  if (k_begin < k_stop) fetch(k_begin);
+  for (int k0 = k_begin; k0 < k_stop; k0 += LM_KEYS) {
     __syncthreads();                                  // the tile before has been read by everyone
     park();
     __syncthreads();
-    if (k0 + LM_KEYS <= p_last) fetch(k0 + LM_KEYS);
+    if (k0 + LM_KEYS < k_stop) fetch(k0 + LM_KEYS);
     // ---- scores of this wavefront's 16 rows against the tile's 32 tokens
     floatx4 sc[2];
 #pragma unroll
@@ -173,6 +183,21 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
       }
     }
   }
+  if (n_splits > 1) {
+    // ---- this share's maximum, sum and unscaled sums: [sequence][row][share][2 + R], merged by another kernel
+    const int rows_cap = gridDim.x * LM_ROWS;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = row0 + wave * 16 + 4 * fg + r;
+      if (row >= T * H) continue;
+      float* pp = partial + (((size_t)blockIdx.y * rows_cap + row) * n_splits + blockIdx.z) * (R + 2);
+      if (fr == 0) { pp[0] = m[r]; pp[1] = l[r]; }
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+        if (i * 16 + fr < R) pp[2 + i * 16 + fr] = o[i][r];
+    }
+    return;
+  }
   // ---- out[token, head, :R] = O / l
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -186,29 +211,83 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   }
 }
 
+// The shares of a row's keys become one: out = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M), shares in ascending order.
+__global__ void attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_splits, const int* __restrict__ q_start,
+                                         int seq0, int H, int R, bf16_t* __restrict__ out, int out_ld) {
+  const int s_local = blockIdx.y, row = blockIdx.x;
+  const int first = q_start[seq0 + s_local], T = q_start[seq0 + s_local + 1] - first;
+  if (row >= T * H) return;
+  const float* pp = partial + ((size_t)s_local * rows_cap + row) * n_splits * (R + 2);
+  float M = -INFINITY;
+  for (int z = 0; z < n_splits; ++z) M = fmaxf(M, pp[(size_t)z * (R + 2)]);
+  float L = 0.f;
+  for (int z = 0; z < n_splits; ++z) {
+    const float mz = pp[(size_t)z * (R + 2)];
+    if (mz != -INFINITY) L += pp[(size_t)z * (R + 2) + 1] * __builtin_amdgcn_exp2f(mz - M);
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  bf16_t* op = out + (size_t)(first + row / H) * out_ld + (size_t)(row % H) * R;
+  for (int c = threadIdx.x; c < R; c += blockDim.x) {
+    float acc = 0.f;
+    for (int z = 0; z < n_splits; ++z) {
+      const float mz = pp[(size_t)z * (R + 2)];
+      if (mz != -INFINITY) acc += pp[(size_t)z * (R + 2) + 2 + c] * __builtin_amdgcn_exp2f(mz - M);
+    }
+    op[c] = f32_to_bf16(acc * inv);
+  }
+}
+
 // Whether the matrix-core form takes these sizes: rows of whole 16-byte pieces, up to the largest form's.
 extern "C" int da_attn_latent_mfma_takes(int D, int R) {
   return D % 8 == 0 && R >= 1 && R <= D && D <= 576 && R <= 512;
 }
 
+// How many workgroups share the keys of a block of query rows when every sequence brings one token (decoding): as
+// many as fill the chip, none with less than two tiles of the longest context that the block table can hold.  From
+// the step's shape only, so that a recorded step keeps it.
+extern "C" int da_attn_latent_splits(int n_seqs, int H, int max_blocks, int page) {
+  const long groups = (long)n_seqs * da_ceil_div(H, LM_ROWS);
+  long n = 384 / (groups > 0 ? groups : 1);
+  const long by_keys = ((long)max_blocks * page) / (2 * LM_KEYS);
+  if (n > by_keys) n = by_keys;
+  if (n > 64) n = 64;
+  return n >= 2 ? (int)n : 1;
+}
+
+extern "C" long da_attn_latent_partial_floats(int S, int max_query_len, int H, int R, int n_splits) {
+  return (long)S * da_ceil_div((long)max_query_len * H, LM_ROWS) * LM_ROWS * n_splits * (R + 2);
+}
+
+// Sequences seq0 .. seq0 + S - 1 of the step.  n_splits > 1: the keys of every block of rows are shared out over
+// that many workgroups, whose results pass through `partial` (32-bit, da_attn_latent_partial_floats entries).
 extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
-                                   const int* q_start, const int* seq_lens, int S, int max_query_len, int H, int D, int R,
-                                   int page, float scale, int window, void* out, int out_ld, void* stream) {
-  DA_REQUIRE(S >= 0 && H > 0 && page > 0 && max_blocks > 0 && max_query_len > 0 && window >= 0, "attn_latent_mfma: bad sizes");
+                                   const int* q_start, const int* seq_lens, int seq0, int S, int max_query_len, int H, int D,
+                                   int R, int page, float scale, int window, void* out, int out_ld, int n_splits,
+                                   float* partial, long partial_floats, void* stream) {
+  DA_REQUIRE(S >= 0 && seq0 >= 0 && H > 0 && page > 0 && max_blocks > 0 && max_query_len > 0 && window >= 0 && n_splits >= 1,
+             "attn_latent_mfma: bad sizes");
   DA_REQUIRE(da_attn_latent_mfma_takes(D, R), "attn_latent_mfma: rows of %d entries with %d of them values are not taken", D, R);
   DA_REQUIRE(q_ld >= H * D && out_ld >= H * R && q_ld % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)cache % 16 == 0,
              "attn_latent_mfma: q must hold H * D entries a row in 16-byte pieces");
+  DA_REQUIRE(n_splits == 1 || (partial && partial_floats >= da_attn_latent_partial_floats(S, max_query_len, H, R, n_splits)),
+             "attn_latent_mfma: the scratch for %d shares is too small", n_splits);
   if (S == 0) return 0;
-  const dim3 grid(da_ceil_div((long)max_query_len * H, LM_ROWS), S), block(256);
+  const dim3 grid(da_ceil_div((long)max_query_len * H, LM_ROWS), S, n_splits), block(256);
   const float sl2 = scale * 1.4426950408889634f;
   hipStream_t st = (hipStream_t)stream;
 #define DA_LM_GO(DB, RB)                                                                                                  \
   hipLaunchKernelGGL((attn_latent_mfma_kernel<DB, RB>), grid, block, 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache,   \
-                     block_table, max_blocks, q_start, seq_lens, H, D, R, page, sl2, window, (bf16_t*)out, out_ld)
+                     block_table, max_blocks, q_start, seq_lens, H, D, R, page, sl2, window, (bf16_t*)out, out_ld, seq0,   \
+                     n_splits, partial)
   if (D <= 128 && R <= 128) DA_LM_GO(4, 8);
   else if (D <= 256 && R <= 256) DA_LM_GO(8, 16);
   else DA_LM_GO(18, 32);
 #undef DA_LM_GO
   DA_CHECK_LAUNCH("attn_latent_mfma");
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(max_query_len * H, S), dim3(128), 0, st, partial, (int)grid.x * LM_ROWS,
+                       n_splits, q_start, seq0, H, R, (bf16_t*)out, out_ld);
+    DA_CHECK_LAUNCH("attn_latent_merge");
+  }
   return 0;
 }

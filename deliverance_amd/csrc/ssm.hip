@@ -143,7 +143,8 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
 #pragma unroll
   for (int j = 0; j < SCAN_SPT; ++j) {
     const bool in_j = j0 + j < n_state;
-    A[j] = in_j ? -expf(load_param(in.a_log, in.a_dtype, (size_t)cc * n_state + j0 + j)) : 0.f;
+    // A = -exp(A_log), times log2(e): the decay exp(dt A) is then one exp2 of the hardware
+    A[j] = in_j ? -expf(load_param(in.a_log, in.a_dtype, (size_t)cc * n_state + j0 + j)) * 1.4426950408889634f : 0.f;
     S[j] = 0.f;
   }
   if (MODE == 0 && slot >= 0) {
@@ -170,7 +171,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
     for (int j = 0; j < SCAN_SPT; ++j) {
       const bool in_j = j0 + j < n_state;
       const float Bj = in_j ? to_f32(bc[in.b_off + j0 + j]) : 0.f;
-      S[j] = expf(dt * A[j]) * S[j] + dx * Bj;
+      S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
       if (MODE != 1) {
         const float Cj = in_j ? to_f32(bc[in.c_off + j0 + j]) : 0.f;
         part = fmaf(S[j], Cj, part);
@@ -214,13 +215,13 @@ __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const f
   const int len = q_start[s + 1] - q_start[s];
   const int n_chunks = (len + chunk - 1) / chunk;
   const int slot = state_slots[s];
-  const float A = -expf(load_param(a_log, a_dtype, i));
+  const float A = -expf(load_param(a_log, a_dtype, i)) * 1.4426950408889634f;
   float S = slot >= 0 ? state[(size_t)slot * state_ld + i] : 0.f;
   for (int k = 0; k < n_chunks; ++k) {
     float* st = chunk_state + ((size_t)s * max_chunks + k) * inner * n_state + i;
     const float own = *st;
     *st = S;
-    S = expf(A * chunk_dt[((size_t)s * max_chunks + k) * inner + c]) * S + own;
+    S = __builtin_amdgcn_exp2f(A * chunk_dt[((size_t)s * max_chunks + k) * inner + c]) * S + own;
   }
   if (slot >= 0 && n_chunks > 0) state[(size_t)slot * state_ld + i] = S;
 }

@@ -115,7 +115,8 @@ _ARGTYPES = {
     "da_rotary": [_VP, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_latent_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP],
     "da_attn_latent_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
-    "da_attn_latent_mfma": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_latent_mfma": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
+    "da_attn_latent_splits": [_I, _I, _I, _I],
     "da_attn_latent_mfma_takes": [_I, _I],
     "da_gemm_heads": [_VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
     "da_gemm_heads_takes": [_I, _I, _I, _I],
@@ -1187,6 +1188,11 @@ def rotary(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, speeds
     return dst
 
 
+def latent_partial_floats(n_seqs: int, max_query_len: int, n_heads: int, v_dim: int, n_splits: int) -> int:
+    """Entries of the 32-bit scratch that the matrix-core latent attention needs to share keys out (blocks of 64 rows)."""
+    return n_seqs * (-(-max_query_len * n_heads // 64)) * 64 * n_splits * (v_dim + 2)
+
+
 def latent_cache_row(cache_slot: torch.Tensor, page: int) -> int:
     """Entries of a row of a latent cache slot [pages, page * D]."""
     return cache_slot[0].numel() // page
@@ -1250,16 +1256,17 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
     el = cache_slot.element_size()
     lens, starts = ctx.seq_lens_host, ctx.q_start_host        # for the profiler's cost model only
 
-    def cost():
+    def cost(first=0, last=None):
         if not KernelProfiler.enabled or not lens:
             return 0, 0
-        keys = pairs = 0
-        for s_ in range(ctx.n_seqs):
+        keys = pairs = rows = 0
+        for s_ in range(first, ctx.n_seqs if last is None else last):
             t = starts[s_ + 1] - starts[s_]
             n = lens[s_]
             keys += n
+            rows += t
             pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
-        return keys * row_dim * el + ctx.n_tokens * n_heads * (row_dim + v_dim) * el, 2 * pairs * n_heads * (row_dim + v_dim)
+        return keys * row_dim * el + rows * n_heads * (row_dim + v_dim) * el, 2 * pairs * n_heads * (row_dim + v_dim)
 
     if (_MODE == "tuned" and q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
             and bool(_lib().da_attn_latent_mfma_takes(row_dim, v_dim))):
@@ -1272,10 +1279,23 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
               "attention_latent: q must be [N, Hq*D] and out [N, Hq*Dv]")
         _need(bt.dtype == torch.int32 and bt.dim() == 2 and bt.is_contiguous() and bt.shape[0] >= ctx.n_seqs,
               "attention_latent: block_table must be contiguous int32 [S, max_blocks]")
-        with _timed("attention_latent", *cost()):
+        nd = ctx.n_decode
+
+        def go(seq0, n_seqs, max_q, n_splits, ws):
             _check(_lib().da_attn_latent_mfma(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(bt), bt.shape[1], _ptr(ctx.q_start),
-                                              _ptr(ctx.seq_lens), ctx.n_seqs, ctx.max_query_len, n_heads, row_dim, v_dim, page,
-                                              float(scale), int(window or 0), _ptr(out), out.stride(0), _stream()))
+                                              _ptr(ctx.seq_lens), seq0, n_seqs, max_q, n_heads, row_dim, v_dim, page,
+                                              float(scale), int(window or 0), _ptr(out), out.stride(0), n_splits, _ptr(ws),
+                                              0 if ws is None else ws.numel(), _stream()))
+        if nd:                 # one-token sequences: the keys of a token's heads shared out over workgroups
+            n_splits = int(_lib().da_attn_latent_splits(nd, n_heads, bt.shape[1], page))
+            ws = None
+            if n_splits > 1:
+                ws = ctx.buf("latent_partial", 1, latent_partial_floats(nd, 1, n_heads, v_dim, n_splits), torch.float32)
+            with _timed("attention_latent_decode", *cost(0, nd)):
+                go(0, nd, 1, n_splits, ws)
+        if ctx.n_seqs > nd:
+            with _timed("attention_latent", *cost(nd, ctx.n_seqs)):
+                go(nd, ctx.n_seqs - nd, ctx.max_query_len, 1, None)
         return out
     with _timed("attention_latent_plain", *cost(), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_latent_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, row_dim, v_dim, page,
@@ -1320,8 +1340,8 @@ def conv_state_update(ctx, x: torch.Tensor, state: torch.Tensor, conv_off: int, 
                                        _ptr(ctx.q_start), ctx.n_seqs, channels, taps, _stream()))
 
 
-SCAN_CHUNK = 64               # tokens of a chunk when a long portion's scan is cut up
-SCAN_CHUNK_FROM = 256         # portions from this length on are cut up
+SCAN_CHUNK = 32               # tokens of a chunk when a long portion's scan is cut up
+SCAN_CHUNK_FROM = 128         # portions from this length on are cut up
 
 
 def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, z: torch.Tensor,

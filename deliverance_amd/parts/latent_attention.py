@@ -58,13 +58,30 @@ class LatentAttention(Mixer):
     def cache_need(self):
         return KVNeed(1, self.row_dim, self.window, self.kv_rank, values_in_keys=True)
 
+    normed_into = True
+
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call, into=None) -> bool:
+        """Small steps: the root-mean-square norm in front and the down-projection in one kernel."""
+        N = x.shape[0]
+        rms = getattr(norm, "rms_params", lambda: None)()
+        if rms is None or not ops.can_fuse_ln(N, x, self.down_weight):
+            return False
+        gain, offset, eps = rms
+        down = ctx.buf("latent_down", N, self.q_rank + self.row_dim, torch.float32)
+        ops.linear_rms(x, None, N, gain, offset, eps, self.down_weight, None, down)
+        self._attend(ctx, down, x if into is None else into, call)
+        return True
+
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
-        N, H = h.shape[0], self.n_heads
+        down = ctx.buf("latent_down", h.shape[0], self.q_rank + self.row_dim, torch.float32)
+        ops.linear(h, self.down_weight, None, down)
+        self._attend(ctx, down, x, call)
+
+    def _attend(self, ctx: StepContext, down: torch.Tensor, x: torch.Tensor, call) -> None:
+        N, H = down.shape[0], self.n_heads
         qd = self.dn + self.dr
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
-        down = ctx.buf("latent_down", N, self.q_rank + self.row_dim, torch.float32)
-        ops.linear(h, self.down_weight, None, down)
         cq = ctx.buf("latent_cq", N, self.q_rank, ctx.dtype)
         ops.latent_prepare(down, self.q_rank, self.kv_rank, self.dr, self.q_gain, self.kv_gain, self.eps, ctx.positions,
                            ctx.slot_maps[group] if call.write else None, self.rotary.speeds, self.rotary.dims,

@@ -44,11 +44,28 @@ class SelectiveScan(Mixer):
     def cache_need(self):
         return StateNeed(self.inner * self.state + (self.taps - 1) * self.inner)
 
+    normed_into = True
+
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call, into=None) -> bool:
+        """Small steps: the root-mean-square norm in front and the up-projection in one kernel."""
+        N = x.shape[0]
+        rms = getattr(norm, "rms_params", lambda: None)()
+        if rms is None or not ops.can_fuse_ln(N, x, self.in_weight):
+            return False
+        gain, offset, eps = rms
+        xz = ctx.buf("scan_xz", N, 2 * self.inner, ctx.dtype)
+        ops.linear_rms(x, None, N, gain, offset, eps, self.in_weight, None, xz)
+        self._scan(ctx, xz, x if into is None else into, call)
+        return True
+
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
-        N, I, n, r = h.shape[0], self.inner, self.state, self.dt_rank
-        state = ctx.cache.state[call.cache]                          # [slots, inner * state + (taps - 1) * inner]
-        xz = ctx.buf("scan_xz", N, 2 * I, ctx.dtype)
+        xz = ctx.buf("scan_xz", h.shape[0], 2 * self.inner, ctx.dtype)
         ops.linear(h, self.in_weight, None, xz)
+        self._scan(ctx, xz, x, call)
+
+    def _scan(self, ctx: StepContext, xz: torch.Tensor, x: torch.Tensor, call) -> None:
+        N, I, n, r = xz.shape[0], self.inner, self.state, self.dt_rank
+        state = ctx.cache.state[call.cache]                          # [slots, inner * state + (taps - 1) * inner]
         xc = ctx.buf("scan_x", N, I, ctx.dtype)
         ops.conv_causal(ctx, xz[:, :I], state, self.conv_off, self.conv_weight, self.conv_bias, "silu", xc)
         if call.write:

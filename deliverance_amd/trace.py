@@ -31,7 +31,7 @@ class TraceSession:
 
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
                  poison_freed: bool = False, kernels: str = "tuned", use_graphs: bool = False, sample: bool = False,
-                 native_step: bool = True, state_slots: int = 4):
+                 native_step: bool = True, state_slots: int = 8):
         import torch
         from . import models  # noqa: F401  (registers the architectures)
         from .config.engine_config import KERNEL_MODES

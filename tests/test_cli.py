@@ -40,6 +40,20 @@ def test_random_then_inspect_another_design(tmp_path):
     assert "l0.mlp.e2.down" in p.stdout and "l2.mlp.table" in p.stdout and "l1.mix.rel" in p.stdout and "[32, 2]" in p.stdout
 
 
+def test_random_then_inspect_a_design_with_shared_weights_and_states(tmp_path):
+    """... and on a Pedatar configuration: layers on another layer's weights store no tensors and keep a cache slot."""
+    from pedatar_models import CONFIG_P
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(CONFIG_P))
+    out = tmp_path / "model"
+    p = run("random", "--config", str(cfg), "--seed", "4", "--out", str(out))
+    assert p.returncode == 0, p.stderr
+    p = run("inspect", str(out))
+    assert p.returncode == 0, p.stderr
+    assert "architecture Pedatar: 2 layers, width 64, vocabulary 300" in p.stdout and "4 layer calls, 4 cache slots" in p.stdout
+    assert "l0.mix.dkv.norm" in p.stdout and "l1.mix.A_log" in p.stdout and "l1.mlp.shared.down" in p.stdout and "l2." not in p.stdout
+
+
 def test_help_names_the_reference_options():
     p = run("generate", "--help")
     for opt in ("--model", "--working-dtype", "--max-tokens", "--temperature", "--seed", "--warmup-cases", "--max-cases",

@@ -212,7 +212,9 @@ def test_latent_attention_finds_one_far_key(dtype, where):
             err = b.step({0: 1})
         else:
             err = b.step({0: T})
-        assert err <= (3e-5 if dtype == "float32" else 3e-2), f"key at {where}, decode={decode}"
+        # (a key that is missed costs an error of the order of the output itself; the bound leaves room for the
+        # roundings of a bfloat16 row that is all one token's value)
+        assert err <= (3e-5 if dtype == "float32" else 6e-2), f"key at {where}, decode={decode}"
     # the case is what it says: the plain weights of the last row put nearly everything on `where`
     W = b.W
     cq = P.unit_rms(b.seqs[0] @ W["mix.dq"].T, W["mix.dq.norm"], 1e-5)
@@ -312,8 +314,8 @@ def test_short_filter_and_state_kernels_alone():
 
 # ------------------------------------------------------------------------------------------ routed feed-forward
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
-@pytest.mark.parametrize("n_experts,top,ff,shared,N", [quick((4, 2, 32, 48, 9)), (1, 1, 40, 0, 5), (3, 3, 20, 0, 70),
-                                                        (12, 3, 24, 16, 300), quick((6, 1, 16, 64, 130))])
+@pytest.mark.parametrize("n_experts,top,ff,shared,N", [quick(4, 2, 32, 48, 9), (1, 1, 40, 0, 5), (3, 3, 20, 0, 70),
+                                                        (12, 3, 24, 16, 300), quick(6, 1, 16, 64, 130)])
 def test_routed_feed_forward_part(n_experts, top, ff, shared, N, dtype):
     """Scores from a logistic router, the best experts, each fed with the row times its score; a shared expert beside
     them.  Few rows (decoding's grouped products) and many (the block tiles with gathered rows)."""

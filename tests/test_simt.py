@@ -33,6 +33,13 @@ RUNS = {
                 "(rms_norm_kernels and 64) or (every_edge and bfloat16) or (experts_feed_forward_part and (64-24 or 300) and bfloat16) "
                 "or (gated_feed_forward_part and 64-40) or (attention_with_bias and bfloat16 and 4-2-16-16) or softcap "
                 "or (whole_prompts and Z and bfloat16)"],
+    # a third design's kernels and parts (rotation, latent attention on its plain and matrix-core forms, the short
+    # filter and the scan, routed experts) and two of its models through the step function
+    "pedatar": ["tests/test_pedatar_gpu.py", "-n", "4"] if FULL else
+               ["tests/test_pedatar_gpu.py", "-n", "3", "-k",
+                "rotation or filter or router_takes or (squared_ramp and bfloat16) or (routed_feed_forward and bfloat16 and not 300) "
+                "or (selective_scan and bfloat16) or (far_key and 31 and bfloat16) or (latent_attention_part and bfloat16 and m0) "
+                "or (whole_prompts and (P or R) and bfloat16) or (mixed_batches and R and bfloat16)"],
     "replay": ["tests/test_replay_gpu.py", "-n", "4"] if FULL else
               ["tests/test_replay_gpu.py", "-n", "2", "-k", "(mixed and (A or B) and not 32) or want_subset or errors_leave or first_tokens"],
     # inner sizes of 32 in an engine step: qkv and fc of seed 11 (and, in the full run, proj of seed 5)
