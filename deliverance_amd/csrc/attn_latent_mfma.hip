@@ -15,6 +15,7 @@
 #define LM_ROWS 64            // query rows a workgroup
 #define LM_KEYS 32            // cached tokens a tile
 #define LM_PAD 8
+#define LM_BT 2048            // entries of a block table that LDS holds
 
 template <int DB, int RB>     // DB: blocks of 32 entries of a cache row (padded), RB: blocks of 16 entries of R
 __global__ void __launch_bounds__(256)
@@ -28,6 +29,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   __shared__ __attribute__((aligned(16))) bf16_t Ks[LM_KEYS * ldk];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * RB * ldv];
   __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * ldv];
+  __shared__ int pages[LM_BT];                        // the sequence's block table (its first LM_BT entries)
 
   const int s = seq0 + blockIdx.y;
   const int first = q_start[s], T = q_start[s + 1] - first;
@@ -38,6 +40,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   const int t = threadIdx.x, lane = t % DA_WAVE, wave = t / DA_WAVE;
   const int fr = lane % 16, fg = lane / 16;
   const int* bt = block_table + (size_t)s * max_blocks;
+  const int page_shift = 31 - __builtin_clz(page);    // (a page holds a power of two of tokens)
 
   // this lane's fragment row, and the four rows whose results it holds
   const int arow = row0 + wave * 16 + fr;
@@ -67,13 +70,19 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
 #pragma unroll
   for (int r = 0; r < 4; ++r) { m[r] = -INFINITY; l[r] = 0.f; }
 
+  // the block table goes to LDS once: a tile's loads then wait for one trip to memory, not for two in a row
+  const int n_bt = (p_last / page + 1 < LM_BT) ? p_last / page + 1 : LM_BT;
+  for (int i = t; i < n_bt; i += 256) pages[i] = bt[i];
   // zero the padding entries of the key tile once (entries D .. D32 of every row)
   for (int i = t; i < LM_KEYS * (D32 - D); i += 256) Ks[(i / (D32 - D)) * ldk + D + i % (D32 - D)] = 0;
   // ... and the rows of the value tile behind R, up to a whole block of 16
   for (int i = t; i < ((R + 15) / 16 * 16 - R) * ldv; i += 256) Vs[R * ldv + i] = 0;
 
   const int chunks = D / 8;                           // 16-byte pieces of a cache row
-  const int n_units = (LM_KEYS / 2) * chunks;         // a unit: the same piece of two neighbouring tokens
+  // a unit: the same piece of two neighbouring tokens.  Neighbouring lanes take neighbouring pairs of tokens, so
+  // that their words of the dimension-major tile lie side by side (lanes along a row's pieces would all meet in
+  // two LDS banks there); four lanes still read 64 consecutive bytes of a row.
+  const int n_units = (LM_KEYS / 2) * chunks;
   constexpr int PER = ((LM_KEYS / 2) * DB * 4 + 255) / 256;
   uint4 stage[PER][2];
   auto fetch = [&](int k0) {
@@ -84,9 +93,10 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
       for (int e = 0; e < 2; ++e) {
         uint4 v = make_uint4(0, 0, 0, 0);
         if (u < n_units) {
-          const int key = k0 + 2 * (u / chunks) + e;
-          const int pg = key <= p_last ? bt[key / page] : -1;     // rows nobody wrote (or gave back) read as zeros
-          if (pg >= 0) v = load16(cache + ((size_t)pg * page + key % page) * D + (u % chunks) * 8);
+          const int key = k0 + 2 * (u % (LM_KEYS / 2)) + e;
+          const int blk = key >> page_shift;
+          const int pg = key <= p_last ? (blk < LM_BT ? pages[blk] : bt[blk]) : -1;     // rows nobody wrote (or gave back) read as zeros
+          if (pg >= 0) v = load16(cache + ((size_t)pg * page + (key & (page - 1))) * D + (u / (LM_KEYS / 2)) * 8);
         }
         stage[i][e] = v;
       }
@@ -97,7 +107,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
     for (int i = 0; i < PER; ++i) {
       const int u = t + i * 256;
       if (u < n_units) {
-        const int kk = 2 * (u / chunks), d = (u % chunks) * 8;
+        const int kk = 2 * (u % (LM_KEYS / 2)), d = (u / (LM_KEYS / 2)) * 8;
         *(uint4*)(Ks + kk * ldk + d) = stage[i][0];
         *(uint4*)(Ks + (kk + 1) * ldk + d) = stage[i][1];
         if (d < R) {                                  // dimension-major: the two tokens' entries side by side, one word
@@ -116,6 +126,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   const int share = (n_tiles + n_splits - 1) / n_splits;
   const int k_begin = key_lo + (int)blockIdx.z * share * LM_KEYS;
   const int k_stop = (k_begin + share * LM_KEYS < p_last + 1) ? k_begin + share * LM_KEYS : p_last + 1;
+  __syncthreads();                                    // the block table's copy is there
   if (k_begin < k_stop) fetch(k_begin);
   for (int k0 = k_begin; k0 < k_stop; k0 += LM_KEYS) {
     __syncthreads();                                  // the tile before has been read by everyone
@@ -212,28 +223,33 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
 }
 
 // The shares of a row's keys become one: out = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M), shares in ascending order.
-__global__ void attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_splits, const int* __restrict__ q_start,
-                                         int seq0, int H, int R, bf16_t* __restrict__ out, int out_ld) {
+#define LM_MAX_SPLITS 64
+__global__ void __launch_bounds__(128)
+attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_splits, const int* __restrict__ q_start,
+                         int seq0, int H, int R, bf16_t* __restrict__ out, int out_ld) {
+  __shared__ float wz[LM_MAX_SPLITS];
   const int s_local = blockIdx.y, row = blockIdx.x;
   const int first = q_start[seq0 + s_local], T = q_start[seq0 + s_local + 1] - first;
   if (row >= T * H) return;
   const float* pp = partial + ((size_t)s_local * rows_cap + row) * n_splits * (R + 2);
-  float M = -INFINITY;
-  for (int z = 0; z < n_splits; ++z) M = fmaxf(M, pp[(size_t)z * (R + 2)]);
-  float L = 0.f;
-  for (int z = 0; z < n_splits; ++z) {
-    const float mz = pp[(size_t)z * (R + 2)];
-    if (mz != -INFINITY) L += pp[(size_t)z * (R + 2) + 1] * __builtin_amdgcn_exp2f(mz - M);
+  if (threadIdx.x < DA_WAVE) {                      // one wavefront: a lane a share
+    const int z = threadIdx.x;
+    const float mz = z < n_splits ? pp[(size_t)z * (R + 2)] : -INFINITY;
+    const float lz = z < n_splits ? pp[(size_t)z * (R + 2) + 1] : 0.f;
+    const float M = wave_max(mz);
+    const float e = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - M);
+    const float L = wave_sum(lz * e);
+    if (z < n_splits) wz[z] = L > 0.f ? e / L : 0.f;
   }
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  __syncthreads();
   bf16_t* op = out + (size_t)(first + row / H) * out_ld + (size_t)(row % H) * R;
   for (int c = threadIdx.x; c < R; c += blockDim.x) {
     float acc = 0.f;
     for (int z = 0; z < n_splits; ++z) {
-      const float mz = pp[(size_t)z * (R + 2)];
-      if (mz != -INFINITY) acc += pp[(size_t)z * (R + 2) + 2 + c] * __builtin_amdgcn_exp2f(mz - M);
+      const float w = wz[z];
+      if (w != 0.f) acc = fmaf(pp[(size_t)z * (R + 2) + 2 + c], w, acc);     // a share without keys holds nothing to read
     }
-    op[c] = f32_to_bf16(acc * inv);
+    op[c] = f32_to_bf16(acc);
   }
 }
 
@@ -250,7 +266,7 @@ extern "C" int da_attn_latent_splits(int n_seqs, int H, int max_blocks, int page
   long n = 384 / (groups > 0 ? groups : 1);
   const long by_keys = ((long)max_blocks * page) / (2 * LM_KEYS);
   if (n > by_keys) n = by_keys;
-  if (n > 64) n = 64;
+  if (n > 16) n = 16;                                 // (every share costs the merge a pass)
   return n >= 2 ? (int)n : 1;
 }
 
@@ -269,6 +285,8 @@ extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, c
   DA_REQUIRE(da_attn_latent_mfma_takes(D, R), "attn_latent_mfma: rows of %d entries with %d of them values are not taken", D, R);
   DA_REQUIRE(q_ld >= H * D && out_ld >= H * R && q_ld % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)cache % 16 == 0,
              "attn_latent_mfma: q must hold H * D entries a row in 16-byte pieces");
+  DA_REQUIRE((page & (page - 1)) == 0, "attn_latent_mfma: a page of %d tokens is no power of two", page);
+  DA_REQUIRE(n_splits <= LM_MAX_SPLITS, "attn_latent_mfma: %d shares, %d are taken", n_splits, LM_MAX_SPLITS);
   DA_REQUIRE(n_splits == 1 || (partial && partial_floats >= da_attn_latent_partial_floats(S, max_query_len, H, R, n_splits)),
              "attn_latent_mfma: the scratch for %d shares is too small", n_splits);
   if (S == 0) return 0;

@@ -10,7 +10,7 @@
 //   da_selective_scan     per channel c and state index j, token by token:
 //                           dt = softplus(raw[n, c]);  S[c, j] = exp(dt * A[c, j]) * S[c, j] + dt * x[n, c] * B[n, j]
 //                           y[n, c] = (sum_j S[c, j] * C[n, j] + D[c] * x[n, c]) * silu(z[n, c])
-//                         with A = -exp(A_log), all in 32-bit; the state is read from the slot at the portion's
+//                         with A = -exp(A_log) (handed over as A log2(e), 32-bit), all in 32-bit; the state is read from the slot at the portion's
 //                         start and written back at its end.
 //   da_scan_chunk_*       the same scan for long portions, cut into chunks that run side by side: each chunk's
 //                         own contribution and decay, then the chunks' starting states one after the other, then
@@ -20,6 +20,8 @@
 #define CONV_MAX_TAPS 16
 #define SCAN_SPT 16          // state entries a thread keeps
 #define SCAN_BLOCK 256
+#define SCAN_TOK 32          // tokens whose B and C wait in LDS together
+#define SCAN_LDS_STATE 64    // state entries of B and of C that LDS holds a token
 
 template <typename T>
 __global__ void conv_causal_kernel(const T* __restrict__ x, int x_ld, const float* __restrict__ state, long state_ld,
@@ -114,7 +116,7 @@ struct ScanIn {
   const void* bc; int bc_ld;          // [N, >= b_off + state], [N, >= c_off + state]
   int b_off, c_off;
   const void* z; int z_ld;            // [N, inner] the gate's input
-  const void* a_log; int a_dtype;     // [inner, state]
+  const float* a2;                    // [inner, state]: A log2(e) = -exp(A_log) log2(e), so that a decay exp(dt A) is one exp2
   const void* d; int d_dtype;         // [inner]
 };
 
@@ -143,8 +145,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
 #pragma unroll
   for (int j = 0; j < SCAN_SPT; ++j) {
     const bool in_j = j0 + j < n_state;
-    // A = -exp(A_log), times log2(e): the decay exp(dt A) is then one exp2 of the hardware
-    A[j] = in_j ? -expf(load_param(in.a_log, in.a_dtype, (size_t)cc * n_state + j0 + j)) * 1.4426950408889634f : 0.f;
+    A[j] = in_j ? in.a2[(size_t)cc * n_state + j0 + j] : 0.f;
     S[j] = 0.f;
   }
   if (MODE == 0 && slot >= 0) {
@@ -160,29 +161,51 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
   }
   const float Dc = in.d ? load_param(in.d, in.d_dtype, cc) : 0.f;
   float dt_sum = 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const size_t n = (size_t)first + t;
-    const float dt = softplus_f32(in.raw[n * in.raw_ld + cc]);
-    const float xv = to_f32(((const T*)in.x)[n * in.x_ld + cc]);
-    const float dx = dt * xv;
-    const T* bc = (const T*)in.bc + n * in.bc_ld;
-    float part = 0.f;
-#pragma unroll
-    for (int j = 0; j < SCAN_SPT; ++j) {
-      const bool in_j = j0 + j < n_state;
-      const float Bj = in_j ? to_f32(bc[in.b_off + j0 + j]) : 0.f;
-      S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
-      if (MODE != 1) {
-        const float Cj = in_j ? to_f32(bc[in.c_off + j0 + j]) : 0.f;
-        part = fmaf(S[j], Cj, part);
+  // B and C of a token are the same for all channels: groups of SCAN_TOK tokens' B | C wait in LDS (up to
+  // SCAN_LDS_STATE entries each; longer ones are read from memory), and a token's own numbers (step size, x, gate)
+  // are asked for one token ahead, so that a step of the recurrence does not wait for memory.
+  __shared__ float bcs[SCAN_TOK][2][SCAN_LDS_STATE];
+  const bool staged = n_state <= SCAN_LDS_STATE;
+  for (int tb = t0; tb < t1; tb += SCAN_TOK) {
+    const int nt = t1 - tb < SCAN_TOK ? t1 - tb : SCAN_TOK;
+    if (staged) {
+      __syncthreads();                                // the group before has been read by everyone
+      for (int i = threadIdx.x; i < nt * 2 * n_state; i += SCAN_BLOCK) {
+        const int tok = i / (2 * n_state), r = i % (2 * n_state), which = r / n_state, j = r % n_state;
+        bcs[tok][which][j] = to_f32(((const T*)in.bc)[((size_t)first + tb + tok) * in.bc_ld + (which ? in.c_off : in.b_off) + j]);
       }
+      __syncthreads();
     }
-    dt_sum += dt;
-    if (MODE != 1) {
-      for (int o = 1; o < L; o <<= 1) part += __shfl_xor(part, o, DA_WAVE);     // the lanes of one channel, fixed order
-      if (live && sub == 0) {
-        const float zv = to_f32(((const T*)in.z)[n * in.z_ld + cc]);
-        from_f32(&y[n * y_ld + cc], (part + Dc * xv) * silu_f32(zv));
+    size_t n = (size_t)first + tb;
+    float raw_n = in.raw[n * in.raw_ld + cc];
+    float x_n = to_f32(((const T*)in.x)[n * in.x_ld + cc]);
+    float z_n = MODE != 1 ? to_f32(((const T*)in.z)[n * in.z_ld + cc]) : 0.f;
+    for (int t = 0; t < nt; ++t) {
+      n = (size_t)first + tb + t;
+      const float raw_c = raw_n, xv = x_n, zv = z_n;
+      const size_t nn = t + 1 < nt ? n + 1 : n;       // the next token's numbers (the last one asks for its own again)
+      raw_n = in.raw[nn * in.raw_ld + cc];
+      x_n = to_f32(((const T*)in.x)[nn * in.x_ld + cc]);
+      if (MODE != 1) z_n = to_f32(((const T*)in.z)[nn * in.z_ld + cc]);
+      const float dt = softplus_f32(raw_c);
+      const float dx = dt * xv;
+      const T* bc = (const T*)in.bc + n * in.bc_ld;
+      float part = 0.f;
+#pragma unroll
+      for (int j = 0; j < SCAN_SPT; ++j) {
+        const bool in_j = j0 + j < n_state;
+        const int jj = in_j ? j0 + j : 0;
+        const float Bj = in_j ? (staged ? bcs[t][0][jj] : to_f32(bc[in.b_off + jj])) : 0.f;
+        S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
+        if (MODE != 1) {
+          const float Cj = in_j ? (staged ? bcs[t][1][jj] : to_f32(bc[in.c_off + jj])) : 0.f;
+          part = fmaf(S[j], Cj, part);
+        }
+      }
+      dt_sum += dt;
+      if (MODE != 1) {
+        for (int o = 1; o < L; o <<= 1) part += __shfl_xor(part, o, DA_WAVE);     // the lanes of one channel, fixed order
+        if (live && sub == 0) from_f32(&y[n * y_ld + cc], (part + Dc * xv) * silu_f32(zv));
       }
     }
   }
@@ -207,7 +230,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
 __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const float* __restrict__ chunk_dt,
                                         int max_chunks, int chunk, float* __restrict__ state, long state_ld,
                                         const int* __restrict__ state_slots, const int* __restrict__ q_start,
-                                        const void* __restrict__ a_log, int a_dtype, int inner, int n_state) {
+                                        const float* __restrict__ a2, int inner, int n_state) {
   const int s = blockIdx.y;
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (long)inner * n_state) return;
@@ -215,7 +238,7 @@ __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const f
   const int len = q_start[s + 1] - q_start[s];
   const int n_chunks = (len + chunk - 1) / chunk;
   const int slot = state_slots[s];
-  const float A = -expf(load_param(a_log, a_dtype, i)) * 1.4426950408889634f;
+  const float A = a2[i];
   float S = slot >= 0 ? state[(size_t)slot * state_ld + i] : 0.f;
   for (int k = 0; k < n_chunks; ++k) {
     float* st = chunk_state + ((size_t)s * max_chunks + k) * inner * n_state + i;
@@ -233,7 +256,7 @@ static int scan_lanes(int n_state) {
 }
 
 extern "C" int da_selective_scan(const void* x, int dtype, int x_ld, const float* raw, int raw_ld, const void* bc, int bc_ld,
-                                 int b_off, int c_off, const void* z, int z_ld, const void* a_log, int a_dtype,
+                                 int b_off, int c_off, const void* z, int z_ld, const float* a2,
                                  const void* d, int d_dtype, float* state, long state_ld, const int* state_slots,
                                  const int* q_start, void* y, int y_ld, int S, int inner, int n_state, int chunk,
                                  int max_chunks, float* chunk_state, float* chunk_dt, void* stream) {
@@ -245,7 +268,7 @@ extern "C" int da_selective_scan(const void* x, int dtype, int x_ld, const float
   DA_REQUIRE(L <= DA_WAVE, "selective_scan: %d state entries a channel, %d are taken", n_state, DA_WAVE * SCAN_SPT);
   DA_REQUIRE(chunk == 0 || (chunk > 0 && max_chunks > 0 && chunk_state && chunk_dt), "selective_scan: chunks need their workspace");
   if (S == 0) return 0;
-  ScanIn in{x, x_ld, raw, raw_ld, bc, bc_ld, b_off, c_off, z, z_ld, a_log, a_dtype, d, d_dtype};
+  ScanIn in{x, x_ld, raw, raw_ld, bc, bc_ld, b_off, c_off, z, z_ld, a2, d, d_dtype};
   hipStream_t st = (hipStream_t)stream;
   const int gx = da_ceil_div((long)inner * L, SCAN_BLOCK);
 #define DA_SCAN_GO(T)                                                                                                        \
@@ -256,8 +279,7 @@ extern "C" int da_selective_scan(const void* x, int dtype, int x_ld, const float
     hipLaunchKernelGGL((selective_scan_kernel<T, 1>), dim3(gx, S, max_chunks), dim3(SCAN_BLOCK), 0, st, in, state, state_ld,  \
                        state_slots, q_start, (T*)y, y_ld, inner, n_state, L, chunk, chunk_state, chunk_dt, max_chunks);       \
     hipLaunchKernelGGL(scan_chunk_carry_kernel, dim3(da_ceil_div((long)inner * n_state, 256), S), dim3(256), 0, st,          \
-                       chunk_state, chunk_dt, max_chunks, chunk, state, state_ld, state_slots, q_start, a_log, a_dtype,      \
-                       inner, n_state);                                                                                      \
+                       chunk_state, chunk_dt, max_chunks, chunk, state, state_ld, state_slots, q_start, a2, inner, n_state);            \
     hipLaunchKernelGGL((selective_scan_kernel<T, 2>), dim3(gx, S, max_chunks), dim3(SCAN_BLOCK), 0, st, in, state, state_ld,  \
                        state_slots, q_start, (T*)y, y_ld, inner, n_state, L, chunk, chunk_state, chunk_dt, max_chunks);       \
   }

@@ -122,7 +122,7 @@ _ARGTYPES = {
     "da_gemm_heads_takes": [_I, _I, _I, _I],
     "da_conv_causal": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
     "da_conv_state_update": [_VP, _I, _I, _VP, ctypes.c_long, _I, _VP, _VP, _I, _I, _I, _VP],
-    "da_selective_scan": [_VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _I, _VP, ctypes.c_long, _VP, _VP,
+    "da_selective_scan": [_VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP, _I, _VP, _VP, _I, _VP, ctypes.c_long, _VP, _VP,
                           _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP],
     "da_moe_combine": [_VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _I, _I, _VP],
 }
@@ -1344,19 +1344,26 @@ SCAN_CHUNK = 32               # tokens of a chunk when a long portion's scan is 
 SCAN_CHUNK_FROM = 128         # portions from this length on are cut up
 
 
+def scan_rates(a_log: torch.Tensor) -> torch.Tensor:
+    """What ``selective_scan`` takes for A = -exp(A_log): A log2(e) in 32-bit, so that a decay exp(dt A) is one exp2."""
+    return (-torch.exp(a_log.to(torch.float32)) * 1.4426950408889634).contiguous()
+
+
 def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, z: torch.Tensor,
-                   a_log: torch.Tensor, d: Optional[torch.Tensor], state: torch.Tensor, y: torch.Tensor, n_state: int) -> torch.Tensor:
-    """The scan of a selective state-space mixer over every sequence of the step (see csrc/ssm.hip); the state
+                   a2: torch.Tensor, d: Optional[torch.Tensor], state: torch.Tensor, y: torch.Tensor, n_state: int) -> torch.Tensor:
+    """The scan of a selective state-space mixer over every sequence of the step (see csrc/ssm.hip), ``a2`` from
+    ``scan_rates``; the state
     [slots, >= inner * n_state] is read at each portion's start and written at its end.  Steps whose longest portion
     has ``SCAN_CHUNK_FROM`` tokens or more are cut into chunks of ``SCAN_CHUNK`` that run side by side."""
-    _dev(x, raw_dt, bc, z, a_log, d, state, y)
+    _dev(x, raw_dt, bc, z, a2, d, state, y)
     for t_, nm in ((x, "x"), (raw_dt, "raw_dt"), (bc, "bc"), (z, "z"), (y, "y")):
         _rows_2d(t_, nm)
     N, inner = y.shape
     ld = _state_args(state, "selective_scan")
     _need(x.shape[0] == N and raw_dt.shape[0] == N and bc.shape[0] == N and z.shape[0] == N, "selective_scan: rows differ")
     _need(raw_dt.dtype == torch.float32 and x.dtype == y.dtype == bc.dtype == z.dtype, "selective_scan: step sizes in float32, the rest of one dtype")
-    _need(a_log.is_contiguous() and tuple(a_log.shape) == (inner, n_state) and (d is None or d.numel() == inner), "selective_scan: A [inner, state], D [inner]")
+    _need(a2.is_contiguous() and a2.dtype == torch.float32 and tuple(a2.shape) == (inner, n_state) and (d is None or d.numel() == inner),
+          "selective_scan: rates float32 [inner, state], D [inner]")
     chunk = max_chunks = 0
     cs = cd = None
     if ctx.max_query_len >= SCAN_CHUNK_FROM:
@@ -1367,7 +1374,7 @@ def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor,
     with _timed("selective_scan", N * inner * (x.element_size() * 3 + 4) + N * 2 * n_state * x.element_size(),
                 N * inner * n_state * 6 * (2 if chunk else 1), "fp32"):
         _check(_lib().da_selective_scan(_ptr(x), _dt(x), x.stride(0), _ptr(raw_dt), raw_dt.stride(0), _ptr(bc), bc.stride(0),
-                                        b_off, c_off, _ptr(z), z.stride(0), _ptr(a_log), _dt(a_log), _ptr(d),
+                                        b_off, c_off, _ptr(z), z.stride(0), _ptr(a2), _ptr(d),
                                         _dt(d) if d is not None else 0, _ptr(state), ld, _ptr(ctx.state_slots), _ptr(ctx.q_start),
                                         _ptr(y), y.stride(0), ctx.n_seqs, inner, n_state, chunk, max_chunks, _ptr(cs), _ptr(cd),
                                         _stream()))

@@ -36,7 +36,8 @@ class SelectiveScan(Mixer):
         self.x_weight = to_matrix(shaped("x_weight", (r + 2 * n, I)), dtype, device)
         self.dt_weight = to_matrix(shaped("dt_weight", (I, r)), dtype, device)
         self.dt_bias = to_vector(shaped("dt_bias", (I,)), dtype, device)
-        self.a_log = to_vector(shaped("a_log", (I, n)), dtype, device)
+        # A = -exp(A_log) in 32-bit, times log2(e) (what the scan kernel takes)
+        self.rates = ops.scan_rates(shaped("a_log", (I, n)).to(device))
         self.d = to_vector(shaped("d", (I,)), dtype, device)
         self.out_weight = to_matrix(shaped("out_weight", (E, I)), dtype, device)
         self.conv_off = I * n                      # where the filter's inputs start in a state row
@@ -75,7 +76,7 @@ class SelectiveScan(Mixer):
         raw = ctx.buf("scan_dt", N, I, torch.float32)                # step sizes before softplus, unrounded
         ops.linear(proj[:, :r], self.dt_weight, self.dt_bias, raw)
         y = ctx.buf("scan_y", N, I, ctx.dtype)
-        ops.selective_scan(ctx, xc, raw, proj, r, r + n, xz[:, I:], self.a_log, self.d, state, y, n)
+        ops.selective_scan(ctx, xc, raw, proj, r, r + n, xz[:, I:], self.rates, self.d, state, y, n)
         ops.linear(y, self.out_weight, None, x, accumulate=ctx.part_accumulate)
 
 
