@@ -48,10 +48,11 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   const bf16_t* qp = q + (size_t)(first + (arow_ok ? arow / H : 0)) * q_ld + (size_t)(arow_ok ? arow % H : 0) * D + fg * 8;
   uint4 qf[DB];
 #pragma unroll
-  for (int i = 0; i < DB; ++i) {
-    const int d = i * 32 + fg * 8;
-    qf[i] = (arow_ok && d < D) ? load16(qp + i * 32) : make_uint4(0, 0, 0, 0);
-  }
+  for (int i = 0; i < DB; ++i)                        // all asked for at once, from places that exist; masked below
+    qf[i] = load16(i * 32 + fg * 8 < D ? qp + i * 32 : qp - fg * 8);
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+    if (!(arow_ok && i * 32 + fg * 8 < D)) qf[i] = make_uint4(0, 0, 0, 0);
   int pos[4];                                         // positions of the rows whose results this lane holds (-1: none)
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -85,34 +86,44 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   const int n_units = (LM_KEYS / 2) * chunks;
   constexpr int PER = ((LM_KEYS / 2) * DB * 4 + 255) / 256;
   uint4 stage[PER][2];
+  unsigned stage_ok = 0;                              // bit 2 i + e: stage[i][e] holds a row that exists
+  // Every load is asked for without a condition, from the row's place or, for a row that does not exist (behind the
+  // last key, or in a page that was given back), from the cache's first row; what came back is looked at only when it
+  // is parked, a tile later.  (A load under a condition, or a value replaced right after its load, makes the
+  // wavefront wait for that load on the spot, one after the other, and nothing would run ahead.)
   auto fetch = [&](int k0) {
+    stage_ok = 0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int u = t + i * 256;
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (u < n_units) {
-          const int key = k0 + 2 * (u % (LM_KEYS / 2)) + e;
-          const int blk = key >> page_shift;
-          const int pg = key <= p_last ? (blk < LM_BT ? pages[blk] : bt[blk]) : -1;     // rows nobody wrote (or gave back) read as zeros
-          if (pg >= 0) v = load16(cache + ((size_t)pg * page + (key & (page - 1))) * D + (u / (LM_KEYS / 2)) * 8);
-        }
-        stage[i][e] = v;
+        const int key = k0 + 2 * (u % (LM_KEYS / 2)) + e;
+        const int blk = key >> page_shift;
+        const bool want = u < n_units && key <= p_last;
+        const int pg = want ? (blk < LM_BT ? pages[blk] : bt[blk]) : -1;
+        const bool ok = pg >= 0;
+        const size_t row = ok ? (size_t)pg * page + (key & (page - 1)) : 0;
+        const int piece = u < n_units ? u / (LM_KEYS / 2) : 0;
+        stage[i][e] = load16(cache + row * D + piece * 8);
+        stage_ok |= (unsigned)ok << (2 * i + e);
       }
     }
   };
   auto park = [&]() {
+    const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int u = t + i * 256;
       if (u < n_units) {
         const int kk = 2 * (u % (LM_KEYS / 2)), d = (u / (LM_KEYS / 2)) * 8;
-        *(uint4*)(Ks + kk * ldk + d) = stage[i][0];
-        *(uint4*)(Ks + (kk + 1) * ldk + d) = stage[i][1];
+        const uint4 v0 = (stage_ok >> (2 * i)) & 1u ? stage[i][0] : zero;      // rows nobody wrote read as zeros
+        const uint4 v1 = (stage_ok >> (2 * i + 1)) & 1u ? stage[i][1] : zero;
+        *(uint4*)(Ks + kk * ldk + d) = v0;
+        *(uint4*)(Ks + (kk + 1) * ldk + d) = v1;
         if (d < R) {                                  // dimension-major: the two tokens' entries side by side, one word
-          const bf16_t* e0 = (const bf16_t*)&stage[i][0];
-          const bf16_t* e1 = (const bf16_t*)&stage[i][1];
+          const bf16_t* e0 = (const bf16_t*)&v0;
+          const bf16_t* e1 = (const bf16_t*)&v1;
 #pragma unroll
           for (int j = 0; j < 8; ++j)
             if (d + j < R) *(uint32_t*)(Vs + (d + j) * ldv + kk) = (uint32_t)e0[j] | ((uint32_t)e1[j] << 16);
@@ -245,10 +256,9 @@ attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_
   bf16_t* op = out + (size_t)(first + row / H) * out_ld + (size_t)(row % H) * R;
   for (int c = threadIdx.x; c < R; c += blockDim.x) {
     float acc = 0.f;
-    for (int z = 0; z < n_splits; ++z) {
-      const float w = wz[z];
-      if (w != 0.f) acc = fmaf(pp[(size_t)z * (R + 2) + 2 + c], w, acc);     // a share without keys holds nothing to read
-    }
+#pragma unroll 4
+    for (int z = 0; z < n_splits; ++z)               // (a share without keys wrote zeros and has the weight 0)
+      acc = fmaf(pp[(size_t)z * (R + 2) + 2 + c], wz[z], acc);
     op[c] = f32_to_bf16(acc);
   }
 }

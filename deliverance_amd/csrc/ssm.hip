@@ -21,6 +21,7 @@
 #define SCAN_SPT 16          // state entries a thread keeps
 #define SCAN_BLOCK 256
 #define SCAN_TOK 32          // tokens whose B and C wait in LDS together
+#define SCAN_GROUP 8         // tokens whose own numbers a thread asks for at once
 #define SCAN_LDS_STATE 64    // state entries of B and of C that LDS holds a token
 
 template <typename T>
@@ -106,8 +107,21 @@ extern "C" int da_conv_state_update(const void* x, int dtype, int x_ld, float* s
   return 0;
 }
 
-__device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+// ln(1 + e^v) and v / (1 + e^-v) with the hardware's exp2, log2 and reciprocal (each within a unit or two in the last
+// place of 32 bits; the library's log1pf and expf cost a hundred instructions a token and channel).  For v below -17
+// the sum 1 + e^v is 1 and the result 0 instead of e^v < 4e-8: a step size that small moves nothing.
+// The 32-bit path (FAST false) keeps the library's functions.
+template <bool FAST>
+__device__ __forceinline__ float softplus_f32(float v) {
+  if (!FAST) return v > 20.f ? v : log1pf(expf(v));
+  const float e = __builtin_amdgcn_exp2f(v * 1.4426950408889634f);
+  return v > 20.f ? v : 0.6931471805599453f * __builtin_amdgcn_logf(1.0f + e);
+}
+template <bool FAST>
+__device__ __forceinline__ float silu_f32(float v) {
+  if (!FAST) return v / (1.0f + expf(-v));
+  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+}
 
 // What a scan kernel reads of the step.
 struct ScanIn {
@@ -141,29 +155,29 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
   const bool live = c < inner;                       // lanes past the last channel follow along and store nothing
   const int cc = live ? c : inner - 1;
   const int j0 = sub * SCAN_SPT;
+  // Every load of the prologue is asked for at once, from a place that exists (an entry past the state's end reads
+  // the row's first one), and looked at afterwards: a load under a condition would be waited for on the spot.
   float A[SCAN_SPT], S[SCAN_SPT];
+  const float* s_from = MODE == 2 ? chunk_state + (((size_t)s * max_chunks + k) * inner + cc) * n_state
+                                  : state + (size_t)(slot >= 0 ? slot : 0) * state_ld + (size_t)cc * n_state;
+  const bool s_given = MODE == 2 || (MODE == 0 && slot >= 0);
+#pragma unroll
+  for (int j = 0; j < SCAN_SPT; ++j) {
+    const int jj = j0 + j < n_state ? j0 + j : 0;
+    A[j] = in.a2[(size_t)cc * n_state + jj];
+    S[j] = MODE == 1 ? 0.f : s_from[jj];
+  }
 #pragma unroll
   for (int j = 0; j < SCAN_SPT; ++j) {
     const bool in_j = j0 + j < n_state;
-    A[j] = in_j ? in.a2[(size_t)cc * n_state + j0 + j] : 0.f;
-    S[j] = 0.f;
-  }
-  if (MODE == 0 && slot >= 0) {
-#pragma unroll
-    for (int j = 0; j < SCAN_SPT; ++j)
-      if (j0 + j < n_state) S[j] = state[(size_t)slot * state_ld + (size_t)cc * n_state + j0 + j];
-  }
-  if (MODE == 2) {
-    const float* st = chunk_state + (((size_t)s * max_chunks + k) * inner + cc) * n_state;
-#pragma unroll
-    for (int j = 0; j < SCAN_SPT; ++j)
-      if (j0 + j < n_state) S[j] = st[j0 + j];
+    A[j] = in_j ? A[j] : 0.f;
+    S[j] = (in_j && s_given) ? S[j] : 0.f;
   }
   const float Dc = in.d ? load_param(in.d, in.d_dtype, cc) : 0.f;
   float dt_sum = 0.f;
   // B and C of a token are the same for all channels: groups of SCAN_TOK tokens' B | C wait in LDS (up to
-  // SCAN_LDS_STATE entries each; longer ones are read from memory), and a token's own numbers (step size, x, gate)
-  // are asked for one token ahead, so that a step of the recurrence does not wait for memory.
+  // SCAN_LDS_STATE entries each; longer ones are read from memory), and the tokens' own numbers (step size, x, gate)
+  // are asked for SCAN_GROUP tokens at a time, so that a step of the recurrence does not wait for memory.
   __shared__ float bcs[SCAN_TOK][2][SCAN_LDS_STATE];
   const bool staged = n_state <= SCAN_LDS_STATE;
   for (int tb = t0; tb < t1; tb += SCAN_TOK) {
@@ -176,36 +190,48 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
       }
       __syncthreads();
     }
-    size_t n = (size_t)first + tb;
-    float raw_n = in.raw[n * in.raw_ld + cc];
-    float x_n = to_f32(((const T*)in.x)[n * in.x_ld + cc]);
-    float z_n = MODE != 1 ? to_f32(((const T*)in.z)[n * in.z_ld + cc]) : 0.f;
-    for (int t = 0; t < nt; ++t) {
-      n = (size_t)first + tb + t;
-      const float raw_c = raw_n, xv = x_n, zv = z_n;
-      const size_t nn = t + 1 < nt ? n + 1 : n;       // the next token's numbers (the last one asks for its own again)
-      raw_n = in.raw[nn * in.raw_ld + cc];
-      x_n = to_f32(((const T*)in.x)[nn * in.x_ld + cc]);
-      if (MODE != 1) z_n = to_f32(((const T*)in.z)[nn * in.z_ld + cc]);
-      const float dt = softplus_f32(raw_c);
-      const float dx = dt * xv;
-      const T* bc = (const T*)in.bc + n * in.bc_ld;
-      float part = 0.f;
+    for (int tg = 0; tg < nt; tg += SCAN_GROUP) {
+      // a group of tokens' own numbers (step size, x, gate) for this thread's channel, all asked for at once
+      float raw_g[SCAN_GROUP], x_g[SCAN_GROUP], z_g[SCAN_GROUP], y_g[SCAN_GROUP];
 #pragma unroll
-      for (int j = 0; j < SCAN_SPT; ++j) {
-        const bool in_j = j0 + j < n_state;
-        const int jj = in_j ? j0 + j : 0;
-        const float Bj = in_j ? (staged ? bcs[t][0][jj] : to_f32(bc[in.b_off + jj])) : 0.f;
-        S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
-        if (MODE != 1) {
-          const float Cj = in_j ? (staged ? bcs[t][1][jj] : to_f32(bc[in.c_off + jj])) : 0.f;
-          part = fmaf(S[j], Cj, part);
+      for (int u = 0; u < SCAN_GROUP; ++u) {
+        const size_t nn = (size_t)first + tb + (tg + u < nt ? tg + u : nt - 1);
+        raw_g[u] = in.raw[nn * in.raw_ld + cc];
+        x_g[u] = to_f32(((const T*)in.x)[nn * in.x_ld + cc]);
+        z_g[u] = MODE != 1 ? to_f32(((const T*)in.z)[nn * in.z_ld + cc]) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < SCAN_GROUP; ++u) {
+        const int t = tg + u;
+        if (t < nt) {                                 // (the same for every thread of the workgroup)
+          const size_t n = (size_t)first + tb + t;
+          const float xv = x_g[u];
+          const float dt = softplus_f32<sizeof(T) == 2>(raw_g[u]);
+          const float dx = dt * xv;
+          const T* bc = (const T*)in.bc + n * in.bc_ld;
+          float part = 0.f;
+#pragma unroll
+          for (int j = 0; j < SCAN_SPT; ++j) {
+            const bool in_j = j0 + j < n_state;
+            const int jj = in_j ? j0 + j : 0;
+            const float Bj = in_j ? (staged ? bcs[t][0][jj] : to_f32(bc[in.b_off + jj])) : 0.f;
+            S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
+            if (MODE != 1) {
+              const float Cj = in_j ? (staged ? bcs[t][1][jj] : to_f32(bc[in.c_off + jj])) : 0.f;
+              part = fmaf(S[j], Cj, part);
+            }
+          }
+          dt_sum += dt;
+          if (MODE != 1) {
+            for (int o = 1; o < L; o <<= 1) part += __shfl_xor(part, o, DA_WAVE);     // the lanes of one channel, fixed order
+            y_g[u] = (part + Dc * xv) * silu_f32<sizeof(T) == 2>(z_g[u]);
+          }
         }
       }
-      dt_sum += dt;
-      if (MODE != 1) {
-        for (int o = 1; o < L; o <<= 1) part += __shfl_xor(part, o, DA_WAVE);     // the lanes of one channel, fixed order
-        if (live && sub == 0) from_f32(&y[n * y_ld + cc], (part + Dc * xv) * silu_f32(zv));
+      if (MODE != 1 && live && sub == 0) {            // the group's results leave together, behind its arithmetic
+#pragma unroll
+        for (int u = 0; u < SCAN_GROUP; ++u)
+          if (tg + u < nt) from_f32(&y[((size_t)first + tb + tg + u) * y_ld + cc], y_g[u]);
       }
     }
   }
