@@ -10,7 +10,7 @@
 //   da_selective_scan     per channel c and state index j, token by token:
 //                           dt = softplus(raw[n, c]);  S[c, j] = exp(dt * A[c, j]) * S[c, j] + dt * x[n, c] * B[n, j]
 //                           y[n, c] = (sum_j S[c, j] * C[n, j] + D[c] * x[n, c]) * silu(z[n, c])
-//                         with A = -exp(A_log) (handed over as A log2(e), 32-bit), all in 32-bit; the state is read from the slot at the portion's
+//                         with A = -exp(A_log) (handed over in 32-bit; times log2(e) for bfloat16 rows), all in 32-bit; the state is read from the slot at the portion's
 //                         start and written back at its end.
 //   da_scan_chunk_*       the same scan for long portions, cut into chunks that run side by side: each chunk's
 //                         own contribution and decay, then the chunks' starting states one after the other, then
@@ -130,7 +130,8 @@ struct ScanIn {
   const void* bc; int bc_ld;          // [N, >= b_off + state], [N, >= c_off + state]
   int b_off, c_off;
   const void* z; int z_ld;            // [N, inner] the gate's input
-  const float* a2;                    // [inner, state]: A log2(e) = -exp(A_log) log2(e), so that a decay exp(dt A) is one exp2
+  const float* a2;                    // [inner, state]: bfloat16 rows: A log2(e) = -exp(A_log) log2(e), so that a decay
+                                      // exp(dt A) is one exp2 of the hardware; 32-bit rows: A itself, and the library's expf
   const void* d; int d_dtype;         // [inner]
 };
 
@@ -215,7 +216,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
             const bool in_j = j0 + j < n_state;
             const int jj = in_j ? j0 + j : 0;
             const float Bj = in_j ? (staged ? bcs[t][0][jj] : to_f32(bc[in.b_off + jj])) : 0.f;
-            S[j] = __builtin_amdgcn_exp2f(dt * A[j]) * S[j] + dx * Bj;
+            S[j] = (sizeof(T) == 2 ? __builtin_amdgcn_exp2f(dt * A[j]) : expf(dt * A[j])) * S[j] + dx * Bj;
             if (MODE != 1) {
               const float Cj = in_j ? (staged ? bcs[t][1][jj] : to_f32(bc[in.c_off + jj])) : 0.f;
               part = fmaf(S[j], Cj, part);
@@ -256,7 +257,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
 __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const float* __restrict__ chunk_dt,
                                         int max_chunks, int chunk, float* __restrict__ state, long state_ld,
                                         const int* __restrict__ state_slots, const int* __restrict__ q_start,
-                                        const float* __restrict__ a2, int inner, int n_state) {
+                                        const float* __restrict__ a2, int inner, int n_state, int fast) {
   const int s = blockIdx.y;
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (long)inner * n_state) return;
@@ -270,7 +271,8 @@ __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const f
     float* st = chunk_state + ((size_t)s * max_chunks + k) * inner * n_state + i;
     const float own = *st;
     *st = S;
-    S = __builtin_amdgcn_exp2f(A * chunk_dt[((size_t)s * max_chunks + k) * inner + c]) * S + own;
+    const float e = A * chunk_dt[((size_t)s * max_chunks + k) * inner + c];
+    S = (fast ? __builtin_amdgcn_exp2f(e) : expf(e)) * S + own;
   }
   if (slot >= 0 && n_chunks > 0) state[(size_t)slot * state_ld + i] = S;
 }
@@ -305,7 +307,7 @@ extern "C" int da_selective_scan(const void* x, int dtype, int x_ld, const float
     hipLaunchKernelGGL((selective_scan_kernel<T, 1>), dim3(gx, S, max_chunks), dim3(SCAN_BLOCK), 0, st, in, state, state_ld,  \
                        state_slots, q_start, (T*)y, y_ld, inner, n_state, L, chunk, chunk_state, chunk_dt, max_chunks);       \
     hipLaunchKernelGGL(scan_chunk_carry_kernel, dim3(da_ceil_div((long)inner * n_state, 256), S), dim3(256), 0, st,          \
-                       chunk_state, chunk_dt, max_chunks, chunk, state, state_ld, state_slots, q_start, a2, inner, n_state);            \
+                       chunk_state, chunk_dt, max_chunks, chunk, state, state_ld, state_slots, q_start, a2, inner, n_state, (int)(sizeof(T) == 2));  \
     hipLaunchKernelGGL((selective_scan_kernel<T, 2>), dim3(gx, S, max_chunks), dim3(SCAN_BLOCK), 0, st, in, state, state_ld,  \
                        state_slots, q_start, (T*)y, y_ld, inner, n_state, L, chunk, chunk_state, chunk_dt, max_chunks);       \
   }

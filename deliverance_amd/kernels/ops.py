@@ -1344,9 +1344,11 @@ SCAN_CHUNK = 32               # tokens of a chunk when a long portion's scan is 
 SCAN_CHUNK_FROM = 128         # portions from this length on are cut up
 
 
-def scan_rates(a_log: torch.Tensor) -> torch.Tensor:
-    """What ``selective_scan`` takes for A = -exp(A_log): A log2(e) in 32-bit, so that a decay exp(dt A) is one exp2."""
-    return (-torch.exp(a_log.to(torch.float32)) * 1.4426950408889634).contiguous()
+def scan_rates(a_log: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """What ``selective_scan`` takes for A = -exp(A_log), in 32-bit: for bfloat16 rows A log2(e), so that a decay
+    exp(dt A) is one exp2 of the hardware; for 32-bit rows A itself (the kernel then calls the library's expf)."""
+    a = -torch.exp(a_log.to(torch.float32))
+    return (a * 1.4426950408889634 if dtype == torch.bfloat16 else a).contiguous()
 
 
 def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, z: torch.Tensor,
@@ -1354,7 +1356,8 @@ def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor,
     """The scan of a selective state-space mixer over every sequence of the step (see csrc/ssm.hip), ``a2`` from
     ``scan_rates``; the state
     [slots, >= inner * n_state] is read at each portion's start and written at its end.  Steps whose longest portion
-    has ``SCAN_CHUNK_FROM`` tokens or more are cut into chunks of ``SCAN_CHUNK`` that run side by side."""
+    has ``SCAN_CHUNK_FROM`` tokens or more are cut into chunks of ``SCAN_CHUNK`` that run side by side (bfloat16 rows;
+    the 32-bit path walks every portion in order, as the recurrence is written)."""
     _dev(x, raw_dt, bc, z, a2, d, state, y)
     for t_, nm in ((x, "x"), (raw_dt, "raw_dt"), (bc, "bc"), (z, "z"), (y, "y")):
         _rows_2d(t_, nm)
@@ -1366,7 +1369,7 @@ def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor,
           "selective_scan: rates float32 [inner, state], D [inner]")
     chunk = max_chunks = 0
     cs = cd = None
-    if ctx.max_query_len >= SCAN_CHUNK_FROM:
+    if ctx.max_query_len >= SCAN_CHUNK_FROM and x.dtype == torch.bfloat16:
         chunk = SCAN_CHUNK
         max_chunks = -(-ctx.max_query_len // chunk)
         cs = ctx.buf("scan_chunk_state", ctx.n_seqs * max_chunks, inner * n_state, torch.float32)

@@ -36,8 +36,8 @@ class SelectiveScan(Mixer):
         self.x_weight = to_matrix(shaped("x_weight", (r + 2 * n, I)), dtype, device)
         self.dt_weight = to_matrix(shaped("dt_weight", (I, r)), dtype, device)
         self.dt_bias = to_vector(shaped("dt_bias", (I,)), dtype, device)
-        # A = -exp(A_log) in 32-bit, times log2(e) (what the scan kernel takes)
-        self.rates = ops.scan_rates(shaped("a_log", (I, n)).to(device))
+        # A = -exp(A_log) in 32-bit (times log2(e) for bfloat16 rows: what the scan kernel takes)
+        self.rates = ops.scan_rates(shaped("a_log", (I, n)).to(device), dtype)
         self.d = to_vector(shaped("d", (I,)), dtype, device)
         self.out_weight = to_matrix(shaped("out_weight", (E, I)), dtype, device)
         self.conv_off = I * n                      # where the filter's inputs start in a state row
