@@ -16,6 +16,7 @@
 //                         own contribution and decay, then the chunks' starting states one after the other, then
 //                         every chunk again from its starting state.
 #include "common.h"
+#include <type_traits>
 
 #define CONV_MAX_TAPS 16
 #define SCAN_SPT 16          // state entries a thread keeps
@@ -179,7 +180,7 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
   // B and C of a token are the same for all channels: groups of SCAN_TOK tokens' B | C wait in LDS (up to
   // SCAN_LDS_STATE entries each; longer ones are read from memory), and the tokens' own numbers (step size, x, gate)
   // are asked for SCAN_GROUP tokens at a time, so that a step of the recurrence does not wait for memory.
-  __shared__ float bcs[SCAN_TOK][2][SCAN_LDS_STATE];
+  __shared__ __attribute__((aligned(16))) float bcs[SCAN_TOK][2][SCAN_LDS_STATE];
   const bool staged = n_state <= SCAN_LDS_STATE;
   for (int tb = t0; tb < t1; tb += SCAN_TOK) {
     const int nt = t1 - tb < SCAN_TOK ? t1 - tb : SCAN_TOK;
@@ -191,41 +192,64 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
       }
       __syncthreads();
     }
-    for (int tg = 0; tg < nt; tg += SCAN_GROUP) {
-      // a group of tokens' own numbers (step size, x, gate) for this thread's channel, all asked for at once
-      float raw_g[SCAN_GROUP], x_g[SCAN_GROUP], z_g[SCAN_GROUP], y_g[SCAN_GROUP];
+    // a group of tokens' own numbers (step size, x, gate) for this thread's channel, all asked for at once, and the
+    // next group's before this group's arithmetic (two sets of registers, taken in turn)
+    float raw_g[2][SCAN_GROUP], x_g[2][SCAN_GROUP], z_g[2][SCAN_GROUP];
+    auto ask = [&](int tg, auto set) {
+      constexpr int b = decltype(set)::value;
 #pragma unroll
       for (int u = 0; u < SCAN_GROUP; ++u) {
         const size_t nn = (size_t)first + tb + (tg + u < nt ? tg + u : nt - 1);
-        raw_g[u] = in.raw[nn * in.raw_ld + cc];
-        x_g[u] = to_f32(((const T*)in.x)[nn * in.x_ld + cc]);
-        z_g[u] = MODE != 1 ? to_f32(((const T*)in.z)[nn * in.z_ld + cc]) : 0.f;
+        raw_g[b][u] = in.raw[nn * in.raw_ld + cc];
+        x_g[b][u] = to_f32(((const T*)in.x)[nn * in.x_ld + cc]);
+        z_g[b][u] = MODE != 1 ? to_f32(((const T*)in.z)[nn * in.z_ld + cc]) : 0.f;
       }
+    };
+    auto group = [&](int tg, auto set) {
+      constexpr int b = decltype(set)::value;
+      if (tg + SCAN_GROUP < nt) ask(tg + SCAN_GROUP, std::integral_constant<int, 1 - b>{});
+      __builtin_amdgcn_sched_barrier(0);              // (asked for here, not where the values are used)
+      float y_g[SCAN_GROUP];
 #pragma unroll
       for (int u = 0; u < SCAN_GROUP; ++u) {
         const int t = tg + u;
         if (t < nt) {                                 // (the same for every thread of the workgroup)
           const size_t n = (size_t)first + tb + t;
-          const float xv = x_g[u];
-          const float dt = softplus_f32<sizeof(T) == 2>(raw_g[u]);
+          const float xv = x_g[b][u];
+          const float dt = softplus_f32<sizeof(T) == 2>(raw_g[b][u]);
           const float dx = dt * xv;
-          const T* bc = (const T*)in.bc + n * in.bc_ld;
+          float Bv[SCAN_SPT], Cv[SCAN_SPT];
+          if (staged) {                               // 16 entries of B and of C in four reads each
+#pragma unroll
+            for (int q4 = 0; q4 < SCAN_SPT / 4; ++q4) {
+              const float4 bq = *(const float4*)&bcs[t][0][j0 + 4 * q4];
+              Bv[4 * q4] = bq.x; Bv[4 * q4 + 1] = bq.y; Bv[4 * q4 + 2] = bq.z; Bv[4 * q4 + 3] = bq.w;
+              if (MODE != 1) {
+                const float4 cq = *(const float4*)&bcs[t][1][j0 + 4 * q4];
+                Cv[4 * q4] = cq.x; Cv[4 * q4 + 1] = cq.y; Cv[4 * q4 + 2] = cq.z; Cv[4 * q4 + 3] = cq.w;
+              }
+            }
+          } else {
+            const T* bc = (const T*)in.bc + n * in.bc_ld;
+#pragma unroll
+            for (int j = 0; j < SCAN_SPT; ++j) {
+              const int jj = j0 + j < n_state ? j0 + j : 0;
+              Bv[j] = to_f32(bc[in.b_off + jj]);
+              if (MODE != 1) Cv[j] = to_f32(bc[in.c_off + jj]);
+            }
+          }
           float part = 0.f;
 #pragma unroll
           for (int j = 0; j < SCAN_SPT; ++j) {
             const bool in_j = j0 + j < n_state;
-            const int jj = in_j ? j0 + j : 0;
-            const float Bj = in_j ? (staged ? bcs[t][0][jj] : to_f32(bc[in.b_off + jj])) : 0.f;
+            const float Bj = in_j ? Bv[j] : 0.f;
             S[j] = (sizeof(T) == 2 ? __builtin_amdgcn_exp2f(dt * A[j]) : expf(dt * A[j])) * S[j] + dx * Bj;
-            if (MODE != 1) {
-              const float Cj = in_j ? (staged ? bcs[t][1][jj] : to_f32(bc[in.c_off + jj])) : 0.f;
-              part = fmaf(S[j], Cj, part);
-            }
+            if (MODE != 1) part = fmaf(S[j], in_j ? Cv[j] : 0.f, part);
           }
           dt_sum += dt;
           if (MODE != 1) {
             for (int o = 1; o < L; o <<= 1) part += __shfl_xor(part, o, DA_WAVE);     // the lanes of one channel, fixed order
-            y_g[u] = (part + Dc * xv) * silu_f32<sizeof(T) == 2>(z_g[u]);
+            y_g[u] = (part + Dc * xv) * silu_f32<sizeof(T) == 2>(z_g[b][u]);
           }
         }
       }
@@ -234,6 +258,11 @@ selective_scan_kernel(ScanIn in, float* __restrict__ state, long state_ld, const
         for (int u = 0; u < SCAN_GROUP; ++u)
           if (tg + u < nt) from_f32(&y[((size_t)first + tb + tg + u) * y_ld + cc], y_g[u]);
       }
+    };
+    ask(0, std::integral_constant<int, 0>{});
+    for (int tg = 0; tg < nt; tg += 2 * SCAN_GROUP) {
+      group(tg, std::integral_constant<int, 0>{});
+      if (tg + SCAN_GROUP < nt) group(tg + SCAN_GROUP, std::integral_constant<int, 1>{});
     }
   }
   if (!live) return;
@@ -267,12 +296,26 @@ __global__ void scan_chunk_carry_kernel(float* __restrict__ chunk_state, const f
   const int slot = state_slots[s];
   const float A = a2[i];
   float S = slot >= 0 ? state[(size_t)slot * state_ld + i] : 0.f;
-  for (int k = 0; k < n_chunks; ++k) {
-    float* st = chunk_state + ((size_t)s * max_chunks + k) * inner * n_state + i;
-    const float own = *st;
-    *st = S;
-    const float e = A * chunk_dt[((size_t)s * max_chunks + k) * inner + c];
-    S = (fast ? __builtin_amdgcn_exp2f(e) : expf(e)) * S + own;
+  for (int k0 = 0; k0 < n_chunks; k0 += 8) {         // eight chunks' numbers asked for at once, then walked in order
+    float own[8], sdt[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int k = k0 + u < n_chunks ? k0 + u : n_chunks - 1;
+      own[u] = chunk_state[((size_t)s * max_chunks + k) * inner * n_state + i];
+      sdt[u] = chunk_dt[((size_t)s * max_chunks + k) * inner + c];
+    }
+    float start[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      start[u] = S;
+      if (k0 + u < n_chunks) {
+        const float e = A * sdt[u];
+        S = (fast ? __builtin_amdgcn_exp2f(e) : expf(e)) * S + own[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (k0 + u < n_chunks) chunk_state[((size_t)s * max_chunks + k0 + u) * inner * n_state + i] = start[u];
   }
   if (slot >= 0 && n_chunks > 0) state[(size_t)slot * state_ld + i] = S;
 }
