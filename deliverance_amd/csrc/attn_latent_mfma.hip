@@ -309,6 +309,7 @@ extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, c
                      n_splits, partial)
   if (D <= 128 && R <= 128) DA_LM_GO(4, 8);
   else if (D <= 256 && R <= 256) DA_LM_GO(8, 16);
+  else if (D <= 384 && R <= 384) DA_LM_GO(12, 24);
   else DA_LM_GO(18, 32);
 #undef DA_LM_GO
   DA_CHECK_LAUNCH("attn_latent_mfma");
