@@ -3,7 +3,8 @@
 //
 //   da_moe_route    from each token's expert ids (read from a table by token id, or given) to a layout in
 //                   which every expert's (token, choice) pairs lie together: pairs get slots, an expert's
-//                   slots start at a multiple of `tile` rows, so that a tile of rows has one expert
+//                   slots start at a multiple of `tile` rows, so that a tile of rows has one expert; weights
+//                   given a pair are also written out a slot
 //   da_moe_gated    mid[slot] = act(Wg_e a[row]) * (Wu_e a[row])      (plain kernel, any dtype)
 //   da_moe_down     out[slot] = Wd_e mid[slot]                        (plain kernel, 32-bit out)
 //   da_moe_combine  y[n] (+)= sum_k weight_k * out[slot(n, k)]        k ascending
@@ -19,7 +20,8 @@
 __global__ void __launch_bounds__(1024)
 moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int vocab, const int* __restrict__ ids,
                  int N, int top, int n_experts, int tile, int* __restrict__ slot_of_pair,
-                 int* __restrict__ row_of_slot, int* __restrict__ tile_expert, int P_cap, int T_cap) {
+                 int* __restrict__ row_of_slot, int* __restrict__ tile_expert, int P_cap, int T_cap,
+                 const float* __restrict__ pair_weights, float* __restrict__ slot_weight) {
   __shared__ int counts[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS], cursor[MOE_MAX_EXPERTS];
   const int t = threadIdx.x, nt = blockDim.x;
   const int P = N * top;
@@ -58,6 +60,7 @@ moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, 
     if (e >= 0) {
       slot = start[e] + atomicAdd(&cursor[e], 1);
       row_of_slot[slot] = i / top;
+      if (pair_weights) slot_weight[slot] = pair_weights[i];      // the pair's weight where its slot's row is
     }
     slot_of_pair[i] = slot;
   }
@@ -65,15 +68,16 @@ moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, 
 
 extern "C" int da_moe_route(const int* tokens, const int* table, int vocab, const int* ids, int N, int top,
                             int n_experts, int tile, int* slot_of_pair, int* row_of_slot, int* tile_expert, int P_cap,
-                            int T_cap, void* stream) {
+                            int T_cap, void* stream, const float* pair_weights, float* slot_weight) {
   DA_REQUIRE(N >= 0 && top > 0 && n_experts > 0 && tile > 0, "moe_route: bad sizes");
   DA_REQUIRE(n_experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, %d are taken", n_experts, MOE_MAX_EXPERTS);
   DA_REQUIRE((table != nullptr && tokens != nullptr) != (ids != nullptr), "moe_route: a table with tokens, or expert ids");
+  DA_REQUIRE((pair_weights == nullptr) == (slot_weight == nullptr), "moe_route: weights a pair need a place a slot");
   DA_REQUIRE(T_cap >= da_ceil_div((long)N * top, tile) + n_experts && P_cap >= T_cap * tile,
              "moe_route: the slot space (%d rows, %d tiles) is too small for %d pairs", P_cap, T_cap, N * top);
   if (N == 0) return 0;
   hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, tokens, table, vocab, ids, N, top,
-                     n_experts, tile, slot_of_pair, row_of_slot, tile_expert, P_cap, T_cap);
+                     n_experts, tile, slot_of_pair, row_of_slot, tile_expert, P_cap, T_cap, pair_weights, slot_weight);
   DA_CHECK_LAUNCH("moe_route");
   return 0;
 }

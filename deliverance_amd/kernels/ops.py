@@ -101,7 +101,7 @@ _ARGTYPES = {
     "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
     "da_softcap": [_VP, ctypes.c_long, _F, _VP],
-    "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP],
+    "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP],
     "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
@@ -365,9 +365,11 @@ def moe_slot_space(n_tokens: int, top: int, n_experts: int, tile: int):
 
 def moe_route(tokens: Optional[torch.Tensor], table: Optional[torch.Tensor], ids: Optional[torch.Tensor], n_tokens: int,
               top: int, n_experts: int, tile: int, slot_of_pair: torch.Tensor, row_of_slot: torch.Tensor,
-              tile_expert: torch.Tensor) -> None:
+              tile_expert: torch.Tensor, pair_weights: Optional[torch.Tensor] = None,
+              slot_weight: Optional[torch.Tensor] = None) -> None:
     """Every (token, choice) pair gets a slot; an expert's slots lie together and start at a multiple of ``tile``.
-    The experts come from ``table[tokens[n], k]`` or from ``ids[n, k]``."""
+    The experts come from ``table[tokens[n], k]`` or from ``ids[n, k]``.  With ``pair_weights`` [N, top] the weight of
+    every pair is also written where its slot is (``slot_weight``, float32, one a slot)."""
     _dev(tokens, table, ids, slot_of_pair, row_of_slot, tile_expert)
     for t_ in (tokens, table, ids, slot_of_pair, row_of_slot, tile_expert):
         _need(t_ is None or (t_.dtype == torch.int32 and t_.is_contiguous()), "moe_route: int32 contiguous operands")
@@ -381,9 +383,16 @@ def moe_route(tokens: Optional[torch.Tensor], table: Optional[torch.Tensor], ids
     tiles, rows = moe_slot_space(n_tokens, top, n_experts, tile)
     _need(slot_of_pair.numel() >= n_tokens * top and row_of_slot.numel() >= rows and tile_expert.numel() >= tiles,
           "moe_route: the outputs are smaller than the slot space")
+    _need((pair_weights is None) == (slot_weight is None), "moe_route: weights a pair need a place a slot")
+    if pair_weights is not None:
+        _dev(pair_weights, slot_weight)
+        _need(pair_weights.dtype == torch.float32 and pair_weights.numel() >= n_tokens * top and pair_weights.is_contiguous()
+              and slot_weight.dtype == torch.float32 and slot_weight.numel() >= rows and slot_weight.is_contiguous(),
+              "moe_route: float32 weights, one a pair and one a slot")
     with _timed("moe_route", 4 * (n_tokens * top * 3 + rows + tiles), 0, "fp32"):
         _check(_lib().da_moe_route(_ptr(tokens), _ptr(table), vocab, _ptr(ids), n_tokens, top, n_experts, tile,
-                                   _ptr(slot_of_pair), _ptr(row_of_slot), _ptr(tile_expert), rows, tiles, _stream()))
+                                   _ptr(slot_of_pair), _ptr(row_of_slot), _ptr(tile_expert), rows, tiles, _stream(),
+                                   _ptr(pair_weights), _ptr(slot_weight)))
 
 
 def _moe_common(a, row_of_slot, tile_expert, w, tiles, tile, name):
@@ -1068,17 +1077,14 @@ def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up
     tiles, rows = moe_slot_space(N, top, n_experts, tile)
     ints = ctx.buf("moe_route", N * top + rows + tiles, 1, torch.int32).view(-1)
     slot_of_pair, row_of_slot, tile_expert = ints[:N * top], ints[N * top:N * top + rows], ints[N * top + rows:]
+    _need(not weight_input or pair_weights is not None, "experts: weights on the input need a weight a pair")
+    # a pair's weight where its slot is: the first product scales its rows with it
+    slot_scale = ctx.buf("moe_slot_scale", rows, 1, torch.float32).view(-1) if weight_input else None
     if ids is None:
         moe_route(ctx.tokens, table, None, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
     else:
-        moe_route(None, None, ids, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert)
-    _need(not weight_input or pair_weights is not None, "experts: weights on the input need a weight a pair")
-    slot_scale = None
-    if weight_input:               # a pair's weight where its slot is: the first product scales its rows with it
-        slot_scale = ctx.buf("moe_slot_scale", rows, 1, torch.float32).view(-1)
-        _dev(pair_weights, slot_scale)
-        _need(pair_weights.dtype == torch.float32 and pair_weights.numel() >= N * top, "experts: a float32 weight a pair")
-        _check(_lib().da_moe_slot_weights(_ptr(slot_of_pair), _ptr(pair_weights), N * top, _ptr(slot_scale), _stream()))
+        moe_route(None, None, ids, N, top, n_experts, tile, slot_of_pair, row_of_slot, tile_expert,
+                  pair_weights if weight_input else None, slot_scale)
     mid = ctx.buf("moe_mid", rows, inner, h.dtype)
     pair_out = ctx.buf("moe_out", rows, width, torch.float32)
     _need(gate_up.is_contiguous() and down.is_contiguous() and tuple(gate_up.shape) == (n_experts, first_rows, width)

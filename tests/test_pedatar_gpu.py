@@ -284,8 +284,8 @@ def test_selective_scan_part_any_cut_and_slots_used_again(m, dtype, monkeypatch)
     step({0: 2, 1: 1})              # shorter than the filter
     step({0: 1, 1: 2, 2: 9})
     step({0: 25, 1: 20})            # chunks of 8: three and a bit, two and a half
-    step({0: 1})
-    step({0: 32, 3: 30})            # slot 0 again, from zero
+    step({0: 1, 3: 22})             # a decoded token beside a portion in chunks; slot 0 again, from zero
+    step({0: 32, 3: 8})
     assert done == [61, 23, 9, 30]
 
 
